@@ -1,0 +1,96 @@
+"""One registry from an architecture's name to the way its model is made.
+
+The reference keys its registry by ``model_type`` and checks the checkpoint's
+``architectures`` against the entry (nanovllm/models/registry.py:36-149); the same
+two keys and the same kinds of error are kept here. An entry is not a model class
+but a recipe: the typed configuration, a function from it to a ``ModelSpec`` (the
+parts of every layer and the run order) and the names of the checkpoint's tensors.
+"""
+from __future__ import annotations
+
+import importlib
+from dataclasses import dataclass
+from typing import Callable
+
+
+class UnknownArchitecture(ValueError):
+    pass
+
+
+@dataclass(frozen=True)
+class WeightSource:
+    """Where one checkpoint tensor goes: into ``param`` (a name of the built model),
+    whole or as rows [row_start, row_start + rows) of a packed parameter."""
+
+    param: str
+    row_start: int = 0
+    rows: int | None = None        # None: the whole parameter
+
+
+@dataclass(frozen=True)
+class Architecture:
+    name: str                                   # e.g. "Qwen3ForCausalLM"
+    model_types: tuple[str, ...]                # values of config.json's model_type
+    parse_config: Callable                      # raw dict -> typed configuration
+    build_spec: Callable                        # typed configuration -> ModelSpec
+    checkpoint_names: Callable                  # typed configuration -> {checkpoint tensor name: WeightSource}
+    optional_names: Callable = lambda cfg: set()  # checkpoint names that may be absent or present
+    ignored_prefixes: tuple[str, ...] = ()      # checkpoint names under these are skipped (nanovllm/utils/loader.py:27-31)
+
+
+_ARCHITECTURES: dict[str, Architecture] = {}
+_LAZY = {
+    # name -> module that registers it on import (nanovllm/models/registry.py:154-159)
+    "Qwen3ForCausalLM": "nanohybrid_vlm_amd.architectures.qwen3",
+}
+_LAZY_MODEL_TYPES = {"qwen3": "Qwen3ForCausalLM"}
+
+
+def register_architecture(arch: Architecture, replace: bool = False) -> None:
+    if arch.name in _ARCHITECTURES and not replace:
+        raise ValueError(f"architecture '{arch.name}' is already registered")
+    _ARCHITECTURES[arch.name] = arch
+
+
+def unregister_architecture(name: str) -> None:
+    _ARCHITECTURES.pop(name, None)
+
+
+def _get(name: str) -> Architecture | None:
+    if name not in _ARCHITECTURES and name in _LAZY:
+        importlib.import_module(_LAZY[name])
+    return _ARCHITECTURES.get(name)
+
+
+def registered_architectures() -> list[str]:
+    return sorted(set(_ARCHITECTURES) | set(_LAZY))
+
+
+def resolve_architecture(raw_config: dict) -> Architecture:
+    """Pick the architecture for a config.json: by ``architectures`` if it lists one
+    that is registered, else by ``model_type``; a ``model_type`` whose entry is not
+    among the listed architectures is an error (registry.py:69-95)."""
+    listed = list(raw_config.get("architectures") or [])
+    model_type = raw_config.get("model_type")
+    for name in listed:
+        arch = _get(name)
+        if arch is not None:
+            if model_type and arch.model_types and model_type not in arch.model_types:
+                raise UnknownArchitecture(
+                    f"config.json: architecture '{name}' does not go with model_type '{model_type}' "
+                    f"(it is registered for {list(arch.model_types)})")
+            return arch
+    if model_type:
+        by_type = [a for a in list(_ARCHITECTURES.values()) if model_type in a.model_types]
+        if not by_type and model_type in _LAZY_MODEL_TYPES:
+            by_type = [_get(_LAZY_MODEL_TYPES[model_type])]
+        if by_type:
+            arch = by_type[0]
+            if listed and arch.name not in listed:
+                raise UnknownArchitecture(
+                    f"config.json: model_type '{model_type}' is registered as '{arch.name}', "
+                    f"but the checkpoint lists {listed}")
+            return arch
+    raise UnknownArchitecture(
+        f"config.json names architectures {listed} and model_type {model_type!r}; "
+        f"registered architectures: {registered_architectures()}")

@@ -1,0 +1,243 @@
+// Embedding gather, RMSNorm (+ residual add), SiLU-and-multiply, row gather and
+// the fused q/k-norm + rotation + cache-write kernel. All in two element types
+// (float, bfloat16); statistics, angles and sums are float.
+#include "nhv_common.h"
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512] = "";
+
+int nhv_fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+extern "C" const char* nhv_last_error() { return g_error; }
+
+// ---------------------------------------------------------------- embedding
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, T* __restrict__ out,
+                             int H, int V) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  const bool ok = id >= 0 && id < V;   // the host checks ids; an id out of range gives a row of zeros, never a wild read
+  const T* src = table + (size_t)(ok ? id : 0) * H;
+  T* dst = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ok ? src[i] : from_f32<T>(0.f);
+}
+
+extern "C" int nhv_embed(const void* ids, const void* table, void* out, int T, int H, int V, int dtype, void* stream) {
+  NHV_REQUIRE(T > 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == NHV_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(T), dim3(256), 0, s, (const int*)ids, (const float*)table, (float*)out, H, V);
+  else if (dtype == NHV_BF16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (const int*)ids, (const bf16_t*)table, (bf16_t*)out, H, V);
+  else
+    return nhv_fail("embed: unknown dtype %d", dtype);
+  NHV_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------- RMSNorm
+// y = round(s * rsqrt(mean(s^2) + eps)) * w in float, s = x or x + residual.
+// residual_mode 0: no residual. 1: s = x + residual, and s replaces the residual.
+// 2: s = x starts a residual (the first norm of a model). The residual may be kept
+// in float while the rows are bfloat16: the sum is then carried unrounded from
+// layer to layer. The weight is multiplied after rounding to the element type, as
+// a separate rounded product.
+template <typename T, typename W, typename R>
+__global__ void rmsnorm_kernel(const T* __restrict__ x, R* __restrict__ residual, int residual_mode,
+                               const W* __restrict__ w, T* __restrict__ y, int H, float eps) {
+  extern __shared__ float row[];          // H floats + 16
+  float* scratch = row + H;
+  const size_t base = (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = to_f32(x[base + i]);
+    if (residual_mode == 1) v += to_f32(residual[base + i]);
+    if (residual_mode != 0) residual[base + i] = from_f32<R>(v);
+    row[i] = v;
+    ss += v * v;
+  }
+  const float total = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(total / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const T n = from_f32<T>(row[i] * r);
+    y[base + i] = from_f32<T>(to_f32(n) * to_f32(w[i]));
+  }
+}
+
+extern "C" int nhv_rmsnorm(const void* x, void* residual, int residual_mode, int residual_dtype, const void* w, void* y,
+                           int T, int H, float eps, int dtype, int w_dtype, void* stream) {
+  NHV_REQUIRE(T > 0 && H > 0, "rmsnorm: bad sizes T=%d H=%d", T, H);
+  NHV_REQUIRE(residual_mode >= 0 && residual_mode <= 2, "rmsnorm: bad residual mode %d", residual_mode);
+  NHV_REQUIRE((residual_mode == 0) == (residual == nullptr), "rmsnorm: residual and its mode do not agree");
+  const size_t lds = ((size_t)H + 16) * sizeof(float);
+  NHV_REQUIRE(lds <= 64 * 1024, "rmsnorm: width %d is beyond this kernel's limit of %d", H, (64 * 1024) / 4 - 16);
+  const int threads = H >= 1024 ? 256 : 64;
+  hipStream_t s = (hipStream_t)stream;
+  if (residual_mode == 0) residual_dtype = NHV_F32;
+#define LAUNCH(TT, WW, RR) \
+  hipLaunchKernelGGL((rmsnorm_kernel<TT, WW, RR>), dim3(T), dim3(threads), lds, s, (const TT*)x, (RR*)residual, residual_mode, (const WW*)w, (TT*)y, H, eps)
+  if (dtype == NHV_F32 && w_dtype == NHV_F32 && residual_dtype == NHV_F32) LAUNCH(float, float, float);
+  else if (dtype == NHV_BF16 && w_dtype == NHV_BF16 && residual_dtype == NHV_F32) LAUNCH(bf16_t, bf16_t, float);
+  else if (dtype == NHV_BF16 && w_dtype == NHV_F32 && residual_dtype == NHV_F32) LAUNCH(bf16_t, float, float);
+  else if (dtype == NHV_BF16 && w_dtype == NHV_BF16 && residual_dtype == NHV_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
+  else if (dtype == NHV_BF16 && w_dtype == NHV_F32 && residual_dtype == NHV_BF16) LAUNCH(bf16_t, float, bf16_t);
+  else return nhv_fail("rmsnorm: unsupported dtypes x=%d w=%d residual=%d", dtype, w_dtype, residual_dtype);
+#undef LAUNCH
+  NHV_LAUNCH_CHECK("rmsnorm");
+  return 0;
+}
+
+// ---------------------------------------------------------------- SiLU(gate) * up
+// gu: [T, 2I], gate = first I columns, up = last I. Float inside, rounded once.
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / I, i = idx % I;
+    const float g = to_f32(gu[t * 2 * I + i]);
+    const float u = to_f32(gu[t * 2 * I + I + i]);
+    out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int nhv_silu_mul(const void* gu, void* out, int T, int I, int dtype, void* stream) {
+  NHV_REQUIRE(T > 0 && I > 0, "silu_mul: bad sizes T=%d I=%d", T, I);
+  const size_t total = (size_t)T * I;
+  const int blocks = (int)((total + 255) / 256 > 65535 * 4 ? 65535 * 4 : (total + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == NHV_F32)
+    hipLaunchKernelGGL(silu_mul_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, total);
+  else if (dtype == NHV_BF16)
+    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, total);
+  else
+    return nhv_fail("silu_mul: unknown dtype %d", dtype);
+  NHV_LAUNCH_CHECK("silu_mul");
+  return 0;
+}
+
+// ---------------------------------------------------------------- row gather
+template <typename T>
+__global__ void gather_rows_kernel(const T* __restrict__ x, const int* __restrict__ rows, T* __restrict__ out,
+                                   int H, int T_in) {
+  int r = rows[blockIdx.x];
+  const bool ok = r >= 0 && r < T_in;
+  const T* src = x + (size_t)(ok ? r : 0) * H;
+  T* dst = out + (size_t)blockIdx.x * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ok ? src[i] : from_f32<T>(0.f);
+}
+
+extern "C" int nhv_gather_rows(const void* x, const void* rows, void* out, int n, int H, int T_in, int dtype, void* stream) {
+  NHV_REQUIRE(n > 0 && H > 0 && T_in > 0, "gather_rows: bad sizes n=%d H=%d T=%d", n, H, T_in);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == NHV_F32)
+    hipLaunchKernelGGL(gather_rows_kernel<float>, dim3(n), dim3(256), 0, s, (const float*)x, (const int*)rows, (float*)out, H, T_in);
+  else if (dtype == NHV_BF16)
+    hipLaunchKernelGGL(gather_rows_kernel<bf16_t>, dim3(n), dim3(256), 0, s, (const bf16_t*)x, (const int*)rows, (bf16_t*)out, H, T_in);
+  else
+    return nhv_fail("gather_rows: unknown dtype %d", dtype);
+  NHV_LAUNCH_CHECK("gather_rows");
+  return 0;
+}
+
+// ---------------------------------------------------------------- q/k norm + rotation + cache write
+// One wave per (token, head) of the packed projection qkv[T, (Hq + 2 Hkv) D]
+// (+ bias). q and k heads: optional RMSNorm over the head (rounded, then times
+// the weight, rounded), then the first `rot` entries are turned pairwise
+// (j, j + rot/2) by the angle of the token's position. q goes to q_out[T, Hq, D];
+// k and v go into the paged cache at slot_mapping[t] (a negative slot is skipped).
+// cos_sin: [max_pos, rot] float, cos in the first rot/2 columns, sin in the rest.
+template <typename T, typename W>
+__global__ void qk_rope_write_kernel(const T* __restrict__ qkv, const T* __restrict__ bias,
+                                     const W* __restrict__ q_norm_w, const W* __restrict__ k_norm_w, float eps,
+                                     const float* __restrict__ cos_sin, int rot,
+                                     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
+                                     T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                     int Hq, int Hkv, int D, int heads_per_token) {
+  extern __shared__ float head[];          // D floats
+  const int t = blockIdx.x / heads_per_token;
+  const int h = blockIdx.x % heads_per_token;
+  const int lane = threadIdx.x;
+  const int width = (Hq + 2 * Hkv) * D;
+  const T* src = qkv + (size_t)t * width + (size_t)h * D;
+  const bool is_q = h < Hq;
+  const bool is_k = !is_q && h < Hq + Hkv;
+  const bool is_v = !is_q && !is_k;
+
+  int slot = -1;
+  if (!is_q) {
+    slot = slot_mapping[t];
+    if (slot < 0) return;                  // whole wave leaves together
+  }
+
+  float ss = 0.f;
+  for (int d = lane; d < D; d += NHV_WAVE) {
+    float v = to_f32(src[d]);
+    if (bias) v = to_f32(from_f32<T>(v + to_f32(bias[(size_t)h * D + d])));
+    head[d] = v;
+    ss += v * v;
+  }
+  if (is_v) {
+    T* dst = v_cache + ((size_t)slot * Hkv + (h - Hq - Hkv)) * D;
+    __builtin_amdgcn_wave_barrier();
+    for (int d = lane; d < D; d += NHV_WAVE) dst[d] = from_f32<T>(head[d]);
+    return;
+  }
+  const W* nw = is_q ? q_norm_w : k_norm_w;
+  if (nw) {
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)D + eps);
+    for (int d = lane; d < D; d += NHV_WAVE) {
+      const T n = from_f32<T>(head[d] * r);
+      head[d] = to_f32(from_f32<T>(to_f32(n) * to_f32(nw[d])));
+    }
+  }
+  __syncthreads();                          // one wave per block: orders the LDS writes before the paired reads
+  T* dst = is_q ? q_out + ((size_t)t * Hq + h) * D : k_cache + ((size_t)slot * Hkv + (h - Hq)) * D;
+  const int half = rot / 2;
+  const float* cs = cos_sin + (size_t)positions[t] * rot;
+  for (int d = lane; d < D; d += NHV_WAVE) {
+    float out;
+    if (d < half) {
+      out = head[d] * cs[d] - head[d + half] * cs[half + d];
+    } else if (d < rot) {
+      const int j = d - half;
+      out = head[d] * cs[j] + head[j] * cs[half + j];
+    } else {
+      out = head[d];
+    }
+    dst[d] = from_f32<T>(out);
+  }
+}
+
+extern "C" int nhv_qk_rope_write(const void* qkv, const void* bias, const void* q_norm_w, const void* k_norm_w, float eps,
+                                 const void* cos_sin, int rot, int max_pos, const void* positions,
+                                 const void* slot_mapping, void* q_out, void* k_cache, void* v_cache, int T, int Hq,
+                                 int Hkv, int D, int write_kv, int dtype, int w_dtype, void* stream) {
+  NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && D > 0, "qk_rope_write: bad sizes T=%d Hq=%d Hkv=%d D=%d", T, Hq, Hkv, D);
+  NHV_REQUIRE(rot >= 0 && rot <= D && rot % 2 == 0, "qk_rope_write: rotary size %d must be even and at most head size %d", rot, D);
+  NHV_REQUIRE(rot == 0 || (cos_sin && max_pos > 0), "qk_rope_write: rotation table missing");
+  NHV_REQUIRE(D <= 4096, "qk_rope_write: head size %d is beyond this kernel's limit of 4096", D);
+  NHV_REQUIRE((q_norm_w == nullptr) == (k_norm_w == nullptr), "qk_rope_write: q and k norm weights come together");
+  NHV_REQUIRE(!write_kv || (slot_mapping && k_cache && v_cache), "qk_rope_write: cache write without cache");
+  const int heads = write_kv ? Hq + 2 * Hkv : Hq;
+  const size_t lds = (size_t)D * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH(TT, WW)                                                                                              \
+  hipLaunchKernelGGL((qk_rope_write_kernel<TT, WW>), dim3((unsigned)((size_t)T * heads)), dim3(NHV_WAVE), lds, s,  \
+                     (const TT*)qkv, (const TT*)bias, (const WW*)q_norm_w, (const WW*)k_norm_w, eps,               \
+                     (const float*)cos_sin, rot, (const int*)positions, (const int*)slot_mapping, (TT*)q_out,       \
+                     (TT*)k_cache, (TT*)v_cache, Hq, Hkv, D, heads)
+  if (dtype == NHV_F32 && w_dtype == NHV_F32) LAUNCH(float, float);
+  else if (dtype == NHV_BF16 && w_dtype == NHV_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (dtype == NHV_BF16 && w_dtype == NHV_F32) LAUNCH(bf16_t, float);
+  else return nhv_fail("qk_rope_write: unsupported dtypes x=%d w=%d", dtype, w_dtype);
+#undef LAUNCH
+  NHV_LAUNCH_CHECK("qk_rope_write");
+  return 0;
+}

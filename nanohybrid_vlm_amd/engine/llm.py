@@ -1,0 +1,233 @@
+"""The Python entry point: ``LLM(model, **options).generate(prompts, sampling_params)``.
+
+Surface and meanings follow the reference (nanovllm/llm.py:4,
+nanovllm/engine/llm_engine.py:176-993): ``add_request``, ``step``, ``is_finished``,
+``generate``, ``exit``; a prompt is a string (needs the checkpoint's tokenizer) or a
+list of token ids; ``generate`` returns ``[{"text", "token_ids"}]`` in the order of
+the prompts. Options are the fields of ``EngineConfig``; an unknown option is an
+error (the reference drops it silently, llm_engine.py:179-181).
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from itertools import count
+from time import perf_counter
+
+from ..config.engine_config import EngineConfig
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler, noise_key
+from .runner import ModelRunner, StepEntry
+from .scheduler import Scheduler
+from .sequence import Sequence
+
+
+@dataclass
+class StepStats:
+    """Tokens and wall time of one step (llm_engine.py:27-63). Decoded tokens and
+    prompt portions run in one pass here, so both rates are over the same time."""
+
+    num_prefill_tokens: int = 0
+    num_decode_tokens: int = 0
+    seconds: float = 0.0
+    num_preempted: int = 0
+
+    @property
+    def prefill_throughput(self) -> float:
+        return self.num_prefill_tokens / self.seconds if self.seconds > 0 else 0.0
+
+    @property
+    def decode_throughput(self) -> float:
+        return self.num_decode_tokens / self.seconds if self.seconds > 0 else 0.0
+
+
+@dataclass
+class RequestMetrics:
+    """Times of one request in seconds of ``perf_counter`` (llm_engine.py:66-174)."""
+
+    seq_id: int
+    num_prompt_tokens: int
+    arrival: float
+    first_scheduled: float | None = None
+    first_token: float | None = None
+    finished: float | None = None
+    num_completion_tokens: int = 0
+
+    @property
+    def ttft_ms(self):
+        return None if self.first_token is None else (self.first_token - self.arrival) * 1e3
+
+    @property
+    def e2e_ms(self):
+        return None if self.finished is None else (self.finished - self.arrival) * 1e3
+
+    @property
+    def tpot_ms(self):
+        if self.finished is None or self.first_token is None or self.num_completion_tokens < 2:
+            return None
+        return (self.finished - self.first_token) * 1e3 / (self.num_completion_tokens - 1)
+
+    @property
+    def queue_ms(self):
+        return None if self.first_scheduled is None else (self.first_scheduled - self.arrival) * 1e3
+
+
+def validate_token_ids(token_ids) -> None:
+    """A non-empty list of non-negative integers (nanovllm/inputs.py:29-55)."""
+    if not isinstance(token_ids, list):
+        raise TypeError("token_ids must be a list")
+    if not token_ids:
+        raise ValueError("token_ids must not be empty")
+    for t in token_ids:
+        if not isinstance(t, int) or isinstance(t, bool):
+            raise TypeError("Every token ID must be an integer")
+        if t < 0:
+            raise ValueError("Token IDs must be non-negative")
+
+
+def _load_tokenizer(folder: str):
+    path = os.path.join(folder, "tokenizer.json")
+    if not os.path.isfile(path):
+        return None
+    from tokenizers import Tokenizer
+    return Tokenizer.from_file(path)
+
+
+class LLM:
+    def __init__(self, model: str, **kwargs):
+        unknown = set(kwargs) - EngineConfig.field_names()
+        if unknown:
+            raise TypeError(f"unknown engine options: {sorted(unknown)}; known: {sorted(EngineConfig.field_names())}")
+        self.config = cfg = EngineConfig(model=model, **kwargs)
+        if not os.path.isdir(model):
+            raise FileNotFoundError(f"model folder '{model}' does not exist")
+        self.runner = ModelRunner(
+            model, dtype=cfg.dtype, page_size=cfg.kvcache_block_size,
+            num_pages=None if cfg.num_kvcache_blocks == -1 else cfg.num_kvcache_blocks,
+            num_state_slots=cfg.max_num_seqs if cfg.num_state_slots == -1 else cfg.num_state_slots,
+            gpu_memory_utilization=cfg.gpu_memory_utilization, max_num_batched_tokens=cfg.max_num_batched_tokens)
+        model_cfg = self.runner.cfg
+        cfg.num_kvcache_blocks = self.runner.num_pages
+        # max_model_len is capped by the model's positions (nanovllm/config.py:420-423)
+        cfg.max_model_len = min(cfg.max_model_len, model_cfg.max_position_embeddings)
+        if cfg.eos == -1 and getattr(model_cfg, "eos_token_id", None) is not None:
+            cfg.eos = model_cfg.eos_token_id
+        self.tokenizer = _load_tokenizer(model)
+        self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.eos,
+                                   cfg.max_model_len, cfg.scheduler_policy, cfg.max_prefill_wait_ms)
+        self.sampler = Sampler(self.runner.vocab_size)
+        self._ids = count()
+        self._sequences: dict[int, Sequence] = {}
+        self._metrics: dict[int, RequestMetrics] = {}
+        self._completed_metrics: list[RequestMetrics] = []
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, prompt, sampling_params: SamplingParams | None = None) -> int:
+        if isinstance(prompt, str):
+            if self.tokenizer is None:
+                raise ValueError("a text prompt needs a tokenizer.json in the model folder; pass token ids instead")
+            token_ids = self.tokenizer.encode(prompt).ids
+        else:
+            validate_token_ids(prompt)
+            token_ids = list(prompt)
+        vocab = self.runner.vocab_size
+        for t in token_ids:
+            if t >= vocab:
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        seq = Sequence(next(self._ids), token_ids, sampling_params)
+        self.scheduler.add(seq)
+        self._sequences[seq.seq_id] = seq
+        self._metrics[seq.seq_id] = RequestMetrics(seq.seq_id, seq.num_prompt_tokens, perf_counter())
+        return seq.seq_id
+
+    def is_finished(self) -> bool:
+        return self.scheduler.is_finished()
+
+    # ------------------------------------------------------------------ one step
+    def step(self):
+        """Plans, runs and finishes one step. Returns ([(seq_id, completion token ids)
+        of the requests that finished], StepStats)."""
+        t0 = perf_counter()
+        plan = self.scheduler.schedule()
+        seqs = plan.seqs
+        entries, sampled_rows = [], []
+        for seq in seqs:
+            n = seq.num_scheduled_tokens
+            start = seq.num_cached_tokens
+            ends = start + n == seq.num_tokens
+            entries.append(StepEntry(seq.seq_id, seq.token_ids[start:start + n], [n - 1] if ends else []))
+            if ends:
+                sampled_rows.append(seq)
+            m = self._metrics[seq.seq_id]
+            if m.first_scheduled is None:
+                m.first_scheduled = t0
+        logits = self.runner.step(entries)
+        tokens_by_id = {}
+        if sampled_rows:
+            seed = self.config.seed
+            temps = [s.temperature for s in sampled_rows]
+            keys = [noise_key(seed if s.seed is None else s.seed, s.seq_id, s.num_completion_tokens)
+                    for s in sampled_rows]
+            tokens = self.sampler(logits, temps, keys)
+            tokens_by_id = {s.seq_id: t for s, t in zip(sampled_rows, tokens)}
+        finished = self.scheduler.postprocess(seqs, [tokens_by_id.get(s.seq_id) for s in seqs])
+        now = perf_counter()
+        for s in sampled_rows:
+            m = self._metrics[s.seq_id]
+            if m.first_token is None:
+                m.first_token = now
+        outputs = []
+        for s in finished:
+            m = self._metrics.pop(s.seq_id)
+            m.finished = now
+            m.num_completion_tokens = s.num_completion_tokens
+            self._completed_metrics.append(m)
+            self._sequences.pop(s.seq_id, None)
+            outputs.append((s.seq_id, s.completion_token_ids))
+        stats = StepStats(num_prefill_tokens=plan.num_prefill_tokens, num_decode_tokens=plan.num_decode_tokens,
+                          seconds=now - t0, num_preempted=len(plan.preempted_seq_ids))
+        return outputs, stats
+
+    # ------------------------------------------------------------------ many prompts
+    def generate(self, prompts: list, sampling_params: SamplingParams | list[SamplingParams],
+                 use_tqdm: bool = True) -> list[dict]:
+        if not isinstance(sampling_params, list):
+            sampling_params = [sampling_params] * len(prompts)
+        if len(sampling_params) != len(prompts):
+            raise ValueError(f"{len(prompts)} prompts but {len(sampling_params)} sampling_params")
+        pbar = None
+        if use_tqdm:
+            from tqdm.auto import tqdm
+            pbar = tqdm(total=len(prompts), desc="Generating", dynamic_ncols=True)
+        ids = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+        outputs = {}
+        prefill_tp = decode_tp = 0.0
+        while not self.is_finished():
+            done, stats = self.step()
+            if stats.num_prefill_tokens:
+                prefill_tp = stats.prefill_throughput
+            if stats.num_decode_tokens:
+                decode_tp = stats.decode_throughput
+            for seq_id, token_ids in done:
+                outputs[seq_id] = token_ids
+                if pbar is not None:
+                    pbar.update(1)
+            if pbar is not None:
+                pbar.set_postfix({"Prefill": f"{int(prefill_tp)}tok/s", "Decode": f"{int(decode_tp)}tok/s"})
+        if pbar is not None:
+            pbar.close()
+        result = []
+        for seq_id in ids:
+            token_ids = outputs[seq_id]
+            text = self.tokenizer.decode(token_ids) if self.tokenizer is not None else None
+            result.append({"text": text, "token_ids": token_ids})
+        return result
+
+    def get_completed_request_metrics(self) -> list[RequestMetrics]:
+        out, self._completed_metrics = self._completed_metrics, []
+        return out
+
+    def exit(self) -> None:
+        """Lets go of the model and the cache."""
+        self.runner = None
+        self.scheduler = None

@@ -1,0 +1,256 @@
+"""The model on the GPU and the one step function.
+
+``ModelRunner`` reads the configuration, builds the model from parts, loads the
+weights, makes the cache (pages per group of layers, state pools per slot) and
+offers ``step``: a batch of (request, its next tokens, the places whose logits are
+wanted). A step runs only the tokens it is given, all requests as one packed
+batch, against what earlier steps left in the cache, and returns float32 logits
+for the wanted places. Prompt portions of any length and single decoded tokens are
+the same kind of entry. Sampling is not done here.
+
+The reference's runner builds two kinds of batch (nanovllm/engine/model_runner.py:
+924-1146) and never mixes them in one forward pass; its index tensors
+(``slot_mapping``, ``block_tables``, ``cu_seqlens_q``, ``context_lens``, positions)
+have the same meaning here.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable
+
+import numpy as np
+import torch
+
+from ..cache.manager import NO_PAGE, CacheManager, PagedGroupSpec
+from ..config.model_config import read_config_json
+from ..config.registry import resolve_architecture
+from ..native.ops import AttentionBatch
+from ..parts.base import CacheView, PagedKVNeed, StateNeed
+from ..parts.context import GroupTables, StepContext
+from ..parts.model import DecoderModel
+from ..weights.loader import load_weights
+
+_TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step."""
+
+    request_id: Hashable
+    tokens: list[int]                       # its next tokens (at least one)
+    want: list[int] = field(default_factory=list)   # places among ``tokens`` whose logits are returned
+
+
+class ModelRunner:
+    def __init__(self, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 256,
+                 num_pages: int | None = None, num_state_slots: int = 512, gpu_memory_utilization: float = 0.9,
+                 max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None):
+        """``model``/``arch``/``cfg`` may be given ready-made (weights already bound)
+        instead of being read from ``model_dir``."""
+        if dtype not in _TORCH_DTYPES:
+            raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
+        self.dtype = _TORCH_DTYPES[dtype]
+        self.device = torch.device(device)
+        if model is None:
+            raw = read_config_json(model_dir)
+            arch = resolve_architecture(raw)
+            cfg = arch.parse_config(raw)
+            model = DecoderModel(arch.build_spec(cfg))
+            load_weights(model, arch, cfg, model_dir, self.dtype, self.device)
+        self.arch, self.cfg, self.model = arch, cfg, model
+        self.model.to(self.device)
+        self.vocab_size = model.spec.vocab_size
+        self.max_position = model.spec.max_position
+        self.page_size = page_size
+        self._make_cache(page_size, num_pages, num_state_slots, gpu_memory_utilization, max_num_batched_tokens)
+        self._pinned = None
+        self._pinned_free = None
+
+    # ------------------------------------------------------------------ cache
+    def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens):
+        needs = self.model.cache_needs()
+        windows: list[int | None] = []                 # one group per distinct window
+        entry_group: dict[int, int] = {}
+        for i, need in enumerate(needs):
+            if isinstance(need, PagedKVNeed):
+                if need.window not in windows:
+                    windows.append(need.window)
+                entry_group[i] = windows.index(need.window)
+        if not windows:
+            windows = [None]                           # a model without paged layers still has one (empty) group
+        item = torch.empty((), dtype=self.dtype).element_size()
+        page_bytes = sum(2 * page_size * n.num_kv_heads * n.head_dim * item
+                         for n in needs if isinstance(n, PagedKVNeed))
+        if num_pages is None:
+            num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens)
+        self.num_pages = num_pages
+        groups = [PagedGroupSpec(name="all keys" if w is None else f"window {w}", page_size=page_size,
+                                 num_pages=num_pages, window=w) for w in windows]
+        self.cache = CacheManager(groups, num_state_slots)
+        views: list[CacheView | None] = [None] * len(needs)
+        self.kv_tensors: list[torch.Tensor] = []
+        self.state_pools: list[dict] = []
+        for i, need in enumerate(needs):
+            if isinstance(need, PagedKVNeed):
+                # [2, pages, page_size, kv_heads, head_dim]: one token's heads lie together
+                # (nanovllm/engine/model_runner.py:870-906)
+                kv = torch.empty((2, num_pages, page_size, need.num_kv_heads, need.head_dim),
+                                 dtype=self.dtype, device=self.device)
+                self.kv_tensors.append(kv)
+                views[i] = CacheView(kind="paged", group=entry_group[i], k=kv[0], v=kv[1], writes=True)
+            elif isinstance(need, StateNeed):
+                pool = {name: torch.zeros((num_state_slots, *shape), dtype=dt, device=self.device)
+                        for name, (shape, dt) in need.tensors.items()}
+                self.state_pools.append(pool)
+                views[i] = CacheView(kind="state", state=pool)
+        for i, e in enumerate(self.model.run_order):
+            if e.cache is not None:
+                lender = views[e.cache]
+                views[i] = CacheView(kind=lender.kind, group=lender.group, k=lender.k, v=lender.v, writes=False,
+                                     state=lender.state)
+            elif views[i] is None:
+                views[i] = CacheView(kind="none")
+        self.model.attach_cache(views)
+
+    def _pages_from_free_memory(self, page_bytes, utilization, max_tokens) -> int:
+        """budget = total * utilization - used - room for a step's activations
+        (nanovllm/engine/model_runner.py:654-699,839-861; the reference measures the
+        room with a warm-up pass, here it is computed from the layer sizes)."""
+        if page_bytes == 0:
+            return 1
+        free, total = torch.cuda.mem_get_info(self.device)
+        s = self.model.spec
+        widest = 0
+        for name, spec in self.model.all_param_specs().items():
+            if len(spec.shape) == 2 and not name.startswith(("embed.", "head.")):
+                widest = max(widest, spec.shape[0])
+        item = torch.empty((), dtype=self.dtype).element_size()
+        activations = max_tokens * (3 * widest + 8 * s.hidden_size) * item + 2 * 512 * s.vocab_size * 4
+        budget = total * utilization - (total - free) - activations
+        pages = int(budget // page_bytes)
+        if pages <= 0:
+            raise RuntimeError(f"no memory left for the cache: {free / 2**30:.1f} GiB free of {total / 2**30:.1f}, "
+                               f"one page needs {page_bytes / 2**20:.1f} MiB")
+        return pages
+
+    # ------------------------------------------------------------------ the step
+    def _stage(self, arrays: list[np.ndarray]) -> list[torch.Tensor]:
+        """All index arrays of a step go to the device in one copy."""
+        sizes = [a.size for a in arrays]
+        total = sum(sizes)
+        if self.device.type == "cuda":
+            if self._pinned is None or self._pinned.numel() < total:
+                self._pinned = torch.empty(max(total, 4096) * 2, dtype=torch.int32, pin_memory=True)
+                self._pinned_free = None
+            if self._pinned_free is not None:
+                self._pinned_free.synchronize()      # the last step's copy has read the buffer
+            host = self._pinned[:total]
+        else:
+            host = torch.empty(total, dtype=torch.int32)
+        flat = host.numpy()
+        offset = 0
+        for a, n in zip(arrays, sizes):
+            flat[offset:offset + n] = a.reshape(-1)
+            offset += n
+        dev = host.to(self.device, non_blocking=True)
+        if self.device.type == "cuda":
+            self._pinned_free = torch.cuda.Event()
+            self._pinned_free.record()
+        out, offset = [], 0
+        for a, n in zip(arrays, sizes):
+            out.append(dev[offset:offset + n].view(a.shape))
+            offset += n
+        return out
+
+    def build_context(self, entries: list[StepEntry]) -> tuple[StepContext, list[int]]:
+        """Reserves pages and lays out the batch. Returns the context and every request's new length."""
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        seen = set()
+        for e in entries:
+            if e.request_id in seen:
+                raise ValueError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.request_id!r}: a step entry needs at least one token")
+        cache = self.cache
+        starts, new_lens = [], []
+        for e in entries:
+            if e.request_id not in cache:
+                cache.admit(e.request_id)
+            start = cache.num_tokens(e.request_id)
+            new_len = start + len(e.tokens)
+            if new_len > self.max_position:
+                raise ValueError(f"request {e.request_id!r}: {new_len} tokens exceed the model's "
+                                 f"{self.max_position} positions")
+            cache.reserve(e.request_id, new_len)
+            starts.append(start)
+            new_lens.append(new_len)
+
+        B = len(entries)
+        q_lens = np.array([len(e.tokens) for e in entries], dtype=np.int32)
+        T = int(q_lens.sum())
+        cu = np.zeros(B + 1, dtype=np.int32)
+        np.cumsum(q_lens, out=cu[1:])
+        input_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        if input_ids.min() < 0 or input_ids.max() >= self.vocab_size:
+            bad = int(input_ids[(input_ids < 0) | (input_ids >= self.vocab_size)][0])
+            raise ValueError(f"token id {bad} is outside the vocabulary of {self.vocab_size}")
+        input_ids = input_ids.astype(np.int32)
+        token_req = np.repeat(np.arange(B, dtype=np.int32), q_lens)
+        positions = (np.arange(T, dtype=np.int32) - np.repeat(cu[:-1], q_lens)
+                     + np.repeat(np.array(starts, dtype=np.int32), q_lens))
+        context_lens = np.array(new_lens, dtype=np.int32)
+        state_slots = np.array([cache.state_slot(e.request_id) for e in entries], dtype=np.int32)
+        rows = []
+        for i, e in enumerate(entries):
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+                rows.append(int(cu[i]) + w)
+        logit_rows = np.array(rows, dtype=np.int32)
+
+        arrays = [input_ids, positions, token_req, cu, context_lens, state_slots, logit_rows]
+        for gi, g in enumerate(cache.groups):
+            tables = [cache.block_table(e.request_id, gi) for e in entries]
+            width = max(1, max(len(t) for t in tables))
+            bt = np.full((B, width), NO_PAGE, dtype=np.int32)
+            slot_mapping = np.empty(T, dtype=np.int32)
+            for i, t in enumerate(tables):
+                ta = np.asarray(t, dtype=np.int32)
+                bt[i, :len(t)] = ta
+                p = positions[cu[i]:cu[i + 1]]
+                pages = ta[p // g.page_size]
+                if (pages == NO_PAGE).any():
+                    raise RuntimeError(f"request {entries[i].request_id!r}: a new token falls on a page that was given back")
+                slot_mapping[cu[i]:cu[i + 1]] = pages * g.page_size + p % g.page_size
+            arrays += [slot_mapping, bt]
+        dev = self._stage(arrays)
+        d_ids, d_pos, d_req, d_cu, d_ctx, d_slots, d_rows = dev[:7]
+        groups = [GroupTables(slot_mapping=dev[7 + 2 * gi], block_tables=dev[8 + 2 * gi])
+                  for gi in range(len(cache.groups))]
+        attention = AttentionBatch(num_tokens=T, num_requests=B, token_req=d_req, positions=d_pos, cu_seqlens_q=d_cu,
+                                   context_lens=d_ctx, max_q_len=int(q_lens.max()), max_context_len=int(max(new_lens)))
+        ctx = StepContext(num_tokens=T, num_requests=B, input_ids=d_ids, positions=d_pos, attention=attention,
+                          groups=groups, state_slots=d_slots, logit_rows=d_rows if len(rows) else None,
+                          num_logit_rows=len(rows),
+                          host={"starts": starts, "new_lens": new_lens, "q_lens": q_lens.tolist(),
+                                "state_slots": state_slots.tolist()})
+        return ctx, new_lens
+
+    @torch.no_grad()
+    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+        """Runs the batch and returns float32 logits [wanted, vocab] in the order of the
+        entries and of each entry's ``want`` (None if nothing is wanted)."""
+        ctx, new_lens = self.build_context(entries)
+        hidden = self.model.forward(ctx)
+        logits = self.model.logits(hidden) if hidden is not None else None
+        for e, n in zip(entries, new_lens):
+            self.cache.commit(e.request_id, n)
+        return logits
+
+    def finish(self, request_id) -> None:
+        """The request is over: its pages and its state slot are given back."""
+        if request_id in self.cache:
+            self.cache.release(request_id)

@@ -1,0 +1,297 @@
+"""The kernels as Python functions over torch tensors on the GPU.
+
+Every function checks on the host that shapes, element types and devices are what
+the kernel and its grid assume, before anything is launched; a size that a kernel
+does not take is refused with an error that names it. Tensors are only memory
+here: the work is done by the HIP library loaded through ``ctypes`` on the
+current torch stream. If the library cannot be built or loaded this raises; there
+is no other implementation behind these functions.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+import torch
+
+from . import library
+
+CORE_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip"]
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    """A kernel refused its arguments or failed to launch."""
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"element type {t.dtype} is not supported (float32 and bfloat16 are)") from None
+
+
+def _ptr(t: torch.Tensor | None):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dense(t: torch.Tensor, name: str, shape: tuple | None = None, dtype=None) -> None:
+    want = backend().device_type
+    _need(t.device.type == want, f"{name}: must live on a '{want}' device, is on {t.device}")
+    _need(t.is_contiguous(), f"{name}: must be contiguous")
+    if shape is not None:
+        _need(tuple(t.shape) == tuple(shape), f"{name}: shape {tuple(t.shape)} but {tuple(shape)} is needed")
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name}: element type {t.dtype} but {dtype} is needed")
+
+
+@dataclass
+class AttentionBatch:
+    """What attention has to know about the step's batch (device tensors are int32)."""
+
+    num_tokens: int
+    num_requests: int
+    token_req: torch.Tensor        # [T] request index of every token
+    positions: torch.Tensor        # [T] absolute position of every token
+    cu_seqlens_q: torch.Tensor     # [B+1] first token of every request in the batch
+    context_lens: torch.Tensor     # [B] keys of the request after this step
+    max_q_len: int
+    max_context_len: int
+
+
+class NativeBackend:
+    """ctypes calls into the HIP library."""
+
+    name = "hip"
+    device_type = "cuda"
+
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible to torch; the HIP kernels are the only implementation")
+        self.lib = library.load_library("nhv_core", CORE_SOURCES)
+        self.lib.nhv_last_error.restype = ctypes.c_char_p
+
+    def _call(self, fn_name: str, *args) -> None:
+        rc = getattr(self.lib, fn_name)(*args)
+        if rc != 0:
+            raise KernelError(self.lib.nhv_last_error().decode())
+
+    # -- each method launches one kernel; arguments were checked by the caller --
+    def embed(self, ids, table, out):
+        T, H = out.shape
+        self._call("nhv_embed", _ptr(ids), _ptr(table), _ptr(out), T, H, table.shape[0], dtype_code(table), _stream())
+
+    def rmsnorm(self, x, residual, residual_mode, w, y, eps):
+        T, H = x.shape
+        self._call("nhv_rmsnorm", _ptr(x), _ptr(residual), residual_mode,
+                   F32 if residual is None else dtype_code(residual), _ptr(w), _ptr(y), T, H, ctypes.c_float(eps),
+                   dtype_code(x), dtype_code(w), _stream())
+
+    def silu_mul(self, gu, out):
+        T, I = out.shape
+        self._call("nhv_silu_mul", _ptr(gu), _ptr(out), T, I, dtype_code(gu), _stream())
+
+    def gather_rows(self, x, rows, out):
+        self._call("nhv_gather_rows", _ptr(x), _ptr(rows), _ptr(out), out.shape[0], x.shape[1], x.shape[0],
+                   dtype_code(x), _stream())
+
+    def qk_rope_write(self, qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, rot, positions, slot_mapping,
+                      q_out, k_cache, v_cache, Hq, Hkv, D, write_kv):
+        wd = dtype_code(q_norm_w) if q_norm_w is not None else dtype_code(qkv)
+        self._call("nhv_qk_rope_write", _ptr(qkv), _ptr(bias), _ptr(q_norm_w), _ptr(k_norm_w), ctypes.c_float(eps),
+                   _ptr(cos_sin), rot, 0 if cos_sin is None else cos_sin.shape[0], _ptr(positions), _ptr(slot_mapping),
+                   _ptr(q_out), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], Hq, Hkv, D, int(write_kv),
+                   dtype_code(qkv), wd, _stream())
+
+    def paged_attention(self, q, k_cache, v_cache, out, batch: AttentionBatch, block_tables, scale, window):
+        T, Hq, D = q.shape
+        _, page_size, Hkv, _ = k_cache.shape
+        self._call("nhv_paged_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
+                   _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables), block_tables.shape[1], T, Hq, Hkv,
+                   D, page_size, ctypes.c_float(scale), window, dtype_code(q), _stream())
+
+    def linear(self, x, w, bias, out):
+        M, K = x.shape
+        N = w.shape[0]
+        self._call("nhv_gemm_generic", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K, dtype_code(x),
+                   dtype_code(out), _stream())
+
+    def sample(self, logits, temperatures, keys, tokens):
+        n, V = logits.shape
+        self._call("nhv_sample", _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(tokens), n, V, _stream())
+
+
+_backend = None
+
+
+def backend():
+    global _backend
+    if _backend is None:
+        _backend = NativeBackend()
+    return _backend
+
+
+def set_backend(obj) -> None:
+    """Replace the kernel library (tests of the engine's logic on a machine
+    without a GPU put a stand-in here; the engine itself never does)."""
+    global _backend
+    _backend = obj
+
+
+# ------------------------------------------------------------------ checked entry points
+def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    _need(table.dim() == 2, "embed: the table must be [vocab, width]")
+    _dense(table, "embed: table")
+    _dense(ids, "embed: ids", (ids.shape[0],), torch.int32)
+    dtype_code(table)
+    out = torch.empty((ids.shape[0], table.shape[1]), dtype=table.dtype, device=table.device)
+    backend().embed(ids, table, out)
+    return out
+
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, residual: torch.Tensor | None = None,
+            start_residual: bool = False):
+    """``rmsnorm(x, w, eps)``: the norm of x.
+    ``residual=r``: r += x in place (in float) and the norm of the sum is returned.
+    ``start_residual=True``: returns (norm of x, a new float32 residual holding x)."""
+    _need(x.dim() == 2, "rmsnorm: x must be [tokens, width]")
+    _dense(x, "rmsnorm: x")
+    _dense(w, "rmsnorm: weight", (x.shape[1],))
+    _need(w.dtype == x.dtype or w.dtype == torch.float32,
+          f"rmsnorm: weight of {w.dtype} with activations of {x.dtype}")
+    dtype_code(x)
+    y = torch.empty_like(x)
+    if start_residual:
+        _need(residual is None, "rmsnorm: a residual is either started or added to")
+        residual = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        backend().rmsnorm(x, residual, 2, w, y, float(eps))
+        return y, residual
+    if residual is not None:
+        _dense(residual, "rmsnorm: residual", tuple(x.shape))
+        _need(residual.dtype == x.dtype or residual.dtype == torch.float32,
+              f"rmsnorm: residual of {residual.dtype} with rows of {x.dtype}")
+        backend().rmsnorm(x, residual, 1, w, y, float(eps))
+        return y
+    backend().rmsnorm(x, None, 0, w, y, float(eps))
+    return y
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "silu_mul: input must be [tokens, 2 * width]")
+    _dense(gate_up, "silu_mul: input")
+    dtype_code(gate_up)
+    out = torch.empty((gate_up.shape[0], gate_up.shape[1] // 2), dtype=gate_up.dtype, device=gate_up.device)
+    backend().silu_mul(gate_up, out)
+    return out
+
+
+def gather_rows(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    _need(x.dim() == 2, "gather_rows: x must be [tokens, width]")
+    _dense(x, "gather_rows: x")
+    _dense(rows, "gather_rows: rows", (rows.shape[0],), torch.int32)
+    dtype_code(x)
+    out = torch.empty((rows.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    backend().gather_rows(x, rows, out)
+    return out
+
+
+def qk_rope_write(qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, positions, slot_mapping, k_cache, v_cache,
+                  num_heads: int, num_kv_heads: int, head_dim: int, write_kv: bool = True) -> torch.Tensor:
+    """Splits the packed projection, norms and turns q and k, stores k and v in the
+    paged cache and returns q as [tokens, heads, head_dim]."""
+    T = qkv.shape[0]
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _dense(qkv, "qk_rope_write: qkv", (T, width))
+    dtype_code(qkv)
+    if bias is not None:
+        _dense(bias, "qk_rope_write: bias", (width,), qkv.dtype)
+    for name, w in (("q_norm", q_norm_w), ("k_norm", k_norm_w)):
+        if w is not None:
+            _dense(w, f"qk_rope_write: {name} weight", (head_dim,))
+            _need(w.dtype == qkv.dtype or w.dtype == torch.float32, f"qk_rope_write: {name} weight of {w.dtype}")
+    _need((q_norm_w is None) == (k_norm_w is None), "qk_rope_write: q and k norm weights come together")
+    if q_norm_w is not None:
+        _need(q_norm_w.dtype == k_norm_w.dtype, "qk_rope_write: q and k norm weights differ in element type")
+    rot = 0
+    if cos_sin is not None:
+        _need(cos_sin.dim() == 2, "qk_rope_write: rotation table must be [positions, rotary size]")
+        _dense(cos_sin, "qk_rope_write: rotation table", dtype=torch.float32)
+        rot = cos_sin.shape[1]
+        _need(rot % 2 == 0 and rot <= head_dim, f"qk_rope_write: rotary size {rot} with head size {head_dim}")
+    _dense(positions, "qk_rope_write: positions", (T,), torch.int32)
+    if write_kv:
+        _dense(slot_mapping, "qk_rope_write: slot_mapping", (T,), torch.int32)
+        _need(k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (num_kv_heads, head_dim),
+              f"qk_rope_write: cache shape {tuple(k_cache.shape)} does not fit {num_kv_heads} heads of {head_dim}")
+        _dense(k_cache, "qk_rope_write: k_cache", dtype=qkv.dtype)
+        _dense(v_cache, "qk_rope_write: v_cache", tuple(k_cache.shape), qkv.dtype)
+    q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    backend().qk_rope_write(qkv, bias, q_norm_w, k_norm_w, float(eps), cos_sin, rot, positions,
+                            slot_mapping if write_kv else None, q_out, k_cache if write_kv else None,
+                            v_cache if write_kv else None, num_heads, num_kv_heads, head_dim, write_kv)
+    return q_out
+
+
+def paged_attention(q, k_cache, v_cache, batch: AttentionBatch, block_tables, scale: float,
+                    window: int | None = None) -> torch.Tensor:
+    _need(q.dim() == 3, "attention: q must be [tokens, heads, head_dim]")
+    T, Hq, D = q.shape
+    _dense(q, "attention: q")
+    dtype_code(q)
+    _need(k_cache.dim() == 4 and k_cache.shape[3] == D, f"attention: cache shape {tuple(k_cache.shape)} with head size {D}")
+    _dense(k_cache, "attention: k_cache", dtype=q.dtype)
+    _dense(v_cache, "attention: v_cache", tuple(k_cache.shape), q.dtype)
+    Hkv = k_cache.shape[2]
+    _need(Hq % Hkv == 0, f"attention: {Hq} query heads are not a multiple of {Hkv} key heads")
+    _need(T == batch.num_tokens, f"attention: {T} tokens but the batch has {batch.num_tokens}")
+    _dense(batch.token_req, "attention: token_req", (T,), torch.int32)
+    _dense(batch.positions, "attention: positions", (T,), torch.int32)
+    _need(block_tables.dim() == 2 and block_tables.shape[0] == batch.num_requests,
+          f"attention: block tables {tuple(block_tables.shape)} for {batch.num_requests} requests")
+    _dense(block_tables, "attention: block_tables", dtype=torch.int32)
+    page_size = k_cache.shape[1]
+    _need(block_tables.shape[1] * page_size >= batch.max_context_len,
+          f"attention: block tables of {block_tables.shape[1]} pages of {page_size} are too short for "
+          f"{batch.max_context_len} keys")
+    out = torch.empty_like(q)
+    backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), int(window or 0))
+    return out
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, out_dtype=None) -> torch.Tensor:
+    """x[M, K] . w[N, K]^T (+ bias), accumulated in float. ``out_dtype`` may be
+    float32 for bfloat16 inputs (the logits)."""
+    _need(x.dim() == 2 and w.dim() == 2, "linear: x must be [rows, in] and w [out, in]")
+    _need(x.shape[1] == w.shape[1], f"linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
+    _dense(x, "linear: x")
+    _dense(w, "linear: w", dtype=x.dtype)
+    dtype_code(x)
+    if bias is not None:
+        _dense(bias, "linear: bias", (w.shape[0],), x.dtype)
+    out_dtype = out_dtype or x.dtype
+    _need(out_dtype == x.dtype or out_dtype == torch.float32, f"linear: output of {out_dtype} from {x.dtype}")
+    out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
+    backend().linear(x, w, bias, out)
+    return out
+
+
+def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:
+    _need(logits.dim() == 2, "sample: logits must be [rows, vocab]")
+    n = logits.shape[0]
+    _dense(logits, "sample: logits", dtype=torch.float32)
+    _dense(temperatures, "sample: temperatures", (n,), torch.float32)
+    _dense(keys, "sample: keys", (n,), torch.int64)
+    tokens = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    backend().sample(logits, temperatures, keys, tokens)
+    return tokens

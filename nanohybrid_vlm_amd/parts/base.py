@@ -1,0 +1,118 @@
+"""What every part of a model is: a thing with sizes given at construction, a list
+of the tensors it needs, and a ``forward`` over the step's packed tokens.
+
+No part reads a model configuration or knows which model it is in: the
+architecture's builder turns the configuration into constructor arguments
+(as the reference's layers take theirs, nanovllm/models/qwen3.py:16-27,93-98).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One tensor that a part needs."""
+
+    shape: tuple[int, ...]
+    init: str = "normal"          # random-weights mode: "normal" N(0, 0.02^2), "norm" 1 + N(0, 0.1^2), "zeros"
+    keeps_float32: bool = False   # a tensor stored in 32-bit stays so even in a bfloat16 run
+
+
+@dataclass(frozen=True)
+class PagedKVNeed:
+    """A mixer that stores a key and a value per token."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None     # None: all keys; n: only the last n are read
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A mixer with state of fixed size per request: name -> (shape of one request's state, dtype)."""
+
+    tensors: dict = field(default_factory=dict)
+
+    def __hash__(self):
+        return hash(tuple(sorted((k, tuple(v[0]), str(v[1])) for k, v in self.tensors.items())))
+
+
+@dataclass
+class CacheView:
+    """The cache that one entry of the run order works on."""
+
+    kind: str                              # "paged" | "state" | "none"
+    group: int = 0                         # paged: which block tables and slot mapping of the step
+    k: torch.Tensor | None = None          # paged: [pages, page_size, kv_heads, head_dim]
+    v: torch.Tensor | None = None
+    writes: bool = True                    # False: the entry reads a cache that another entry fills
+    state: dict | None = None              # state: name -> [slots, ...]
+
+
+class Part:
+    """Base of mixers, feed-forwards, norms, position encodings and blocks."""
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {}
+
+    def children(self) -> dict[str, "Part"]:
+        return {}
+
+    def bind(self, params: dict[str, torch.Tensor]) -> None:
+        """Receives this part's own tensors (names as in ``param_specs``)."""
+        for name, tensor in params.items():
+            setattr(self, name.replace(".", "_"), tensor)
+
+    # -- walking the tree -------------------------------------------------
+    def all_param_specs(self, prefix: str = "") -> dict[str, ParamSpec]:
+        out = {prefix + k: v for k, v in self.param_specs().items()}
+        for cname, child in self.children().items():
+            out.update(child.all_param_specs(f"{prefix}{cname}."))
+        return out
+
+    def bind_all(self, params: dict[str, torch.Tensor], prefix: str = "") -> None:
+        own = {k: params[prefix + k] for k in self.param_specs()}
+        self.bind(own)
+        for cname, child in self.children().items():
+            child.bind_all(params, f"{prefix}{cname}.")
+
+
+class Registry:
+    """Name -> constructor for one kind of part."""
+
+    def __init__(self, what: str):
+        self.what = what
+        self._makers: dict[str, Callable] = {}
+
+    def register(self, kind: str):
+        def deco(maker):
+            if kind in self._makers:
+                raise ValueError(f"{self.what} '{kind}' is already registered")
+            self._makers[kind] = maker
+            return maker
+        return deco
+
+    def unregister(self, kind: str) -> None:
+        self._makers.pop(kind, None)
+
+    def kinds(self) -> list[str]:
+        return sorted(self._makers)
+
+    def build(self, spec: dict, **extra):
+        """``spec`` = {"kind": name, ...constructor arguments}."""
+        spec = dict(spec)
+        kind = spec.pop("kind", None)
+        if kind not in self._makers:
+            raise KeyError(f"unknown {self.what} '{kind}'; registered: {self.kinds()}")
+        return self._makers[kind](**spec, **extra)
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+BLOCKS = Registry("block")

@@ -1,0 +1,143 @@
+"""A decoder as data, and the one class that runs any such description.
+
+``ModelSpec`` says which parts every layer is made of and in which order layers
+run. ``DecoderModel`` builds the parts through the registries and runs them over
+the step's packed tokens. An architecture is a function from its configuration to
+a ``ModelSpec`` plus the names of its checkpoint tensors (``config/registry.py``).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..native import ops
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheView, PagedKVNeed, ParamSpec, Part,
+                   StateNeed)
+
+
+@dataclass
+class LayerSpec:
+    """One layer: each entry is {"kind": registered name, ...constructor arguments}."""
+
+    mixer: dict
+    feed_forward: dict
+    norm: dict
+    block: dict = field(default_factory=lambda: {"kind": "prenorm"})
+    position: str | None = "default"      # name in ModelSpec.positions that the mixer gets, or None
+
+
+@dataclass
+class RunEntry:
+    """One step of the run order. ``cache`` names the entry (by its index in the run
+    order) whose cache this entry reads without writing; None: the entry has a
+    cache of its own and fills it."""
+
+    layer: int
+    cache: int | None = None
+
+
+@dataclass
+class ModelSpec:
+    vocab_size: int
+    hidden_size: int
+    layers: list[LayerSpec]
+    final_norm: dict
+    positions: dict                        # name -> {"kind": ..., ...}; layers refer to these by name
+    max_position: int
+    tie_embeddings: bool
+    run_order: list[RunEntry] | None = None   # None: every layer once, in order
+
+    def order(self) -> list[RunEntry]:
+        if self.run_order is None:
+            return [RunEntry(i) for i in range(len(self.layers))]
+        return self.run_order
+
+
+class DecoderModel(Part):
+    """Embedding, the layers in run order, final norm, and the head on the wanted rows."""
+
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.positions = {name: POSITION_ENCODINGS.build(p, max_position=spec.max_position)
+                          for name, p in spec.positions.items()}
+        self.layers = []
+        for ls in spec.layers:
+            mixer_args = {}
+            if ls.position is not None:
+                mixer_args["position"] = self.positions[ls.position]
+            mixer = MIXERS.build(ls.mixer, **mixer_args)
+            ff = FEED_FORWARDS.build(ls.feed_forward)
+            block = BLOCKS.build(ls.block, mixer=mixer, feed_forward=ff,
+                                 mixer_norm=NORMS.build(ls.norm), feed_forward_norm=NORMS.build(ls.norm))
+            self.layers.append(block)
+        self.final_norm = NORMS.build(spec.final_norm)
+        self.run_order = spec.order()
+        for i, e in enumerate(self.run_order):
+            if not 0 <= e.layer < len(self.layers):
+                raise ValueError(f"run order entry {i} names layer {e.layer}; there are {len(self.layers)}")
+            if e.cache is not None:
+                if not 0 <= e.cache < i or self.run_order[e.cache].cache is not None:
+                    raise ValueError(f"run order entry {i} reads the cache of entry {e.cache}, which must be an "
+                                     f"earlier entry with a cache of its own")
+                if self.layers[e.layer].mixer.cache_need() != self.layers[self.run_order[e.cache].layer].mixer.cache_need():
+                    raise ValueError(f"run order entry {i} and entry {e.cache} need different caches")
+        self.embed_weight = None
+        self.head_weight = None
+        self.cache_views: list[CacheView] = []
+
+    # -- parameters -------------------------------------------------------
+    def param_specs(self):
+        s = self.spec
+        specs = {"embed.weight": ParamSpec((s.vocab_size, s.hidden_size))}
+        if not s.tie_embeddings:
+            specs["head.weight"] = ParamSpec((s.vocab_size, s.hidden_size))
+        return specs
+
+    def children(self):
+        out = {f"layers.{i}": layer for i, layer in enumerate(self.layers)}
+        out["final_norm"] = self.final_norm
+        return out
+
+    def bind(self, params):
+        self.embed_weight = params["embed.weight"]
+        # tied: the head reads the embedding's own storage (nanovllm/models/qwen3.py:202-203)
+        self.head_weight = params["embed.weight"] if self.spec.tie_embeddings else params["head.weight"]
+
+    def to(self, device):
+        for p in self.positions.values():
+            p.to(device)
+        return self
+
+    # -- cache ------------------------------------------------------------
+    def cache_needs(self) -> list[PagedKVNeed | StateNeed | None]:
+        """Per run-order entry: what cache of its own it needs (None when it has none or borrows one)."""
+        out = []
+        for e in self.run_order:
+            out.append(self.layers[e.layer].mixer.cache_need() if e.cache is None else None)
+        return out
+
+    def attach_cache(self, views: list[CacheView]) -> None:
+        """``views[i]`` is the cache of run-order entry i (for a borrowing entry: the lender's, with writes off)."""
+        if len(views) != len(self.run_order):
+            raise ValueError(f"{len(views)} cache views for {len(self.run_order)} run-order entries")
+        self.cache_views = views
+
+    # -- the forward pass -------------------------------------------------
+    def forward(self, step) -> torch.Tensor:
+        """Hidden states after the final norm, for the rows whose logits are wanted only: [n, hidden]."""
+        hidden = ops.embed(step.input_ids, self.embed_weight)
+        residual = None
+        for entry, cache in zip(self.run_order, self.cache_views):
+            hidden, residual = self.layers[entry.layer].forward(hidden, residual, step, cache)
+        if step.num_logit_rows == 0:
+            return None
+        # only the wanted rows go through the last norm and the head (nanovllm/layers/embed_head.py:56-61)
+        hidden = ops.gather_rows(hidden, step.logit_rows)
+        residual = ops.gather_rows(residual, step.logit_rows)
+        hidden, _ = self.final_norm.forward_add(hidden, residual)
+        return hidden
+
+    def logits(self, hidden: torch.Tensor) -> torch.Tensor:
+        """float32 logits [n, vocab] (the reference's sampler casts to float first, nanovllm/layers/sampler.py:12)."""
+        return ops.linear(hidden, self.head_weight, out_dtype=torch.float32)

@@ -1,0 +1,335 @@
+"""Every HIP kernel alone against a plain torch float32 reference of the same
+operation, at sizes other than the tiny models' (widths and vocabularies that are
+no power of two, odd head counts, head sizes in steps of 16, page sizes that do not
+divide the lengths). Pure data movement must be bit-exact."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    # float32: rounding of a few float operations; bfloat16: one rounding to 8 bits (2^-9 relative) of
+    # values of size about 1-4
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1.6e-2)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from nanohybrid_vlm_amd.native import ops as o
+    assert o.backend().name == "hip"
+    return o
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H,V", [(1, 80, 301), (37, 1000, 77), (300, 4096, 1000)])
+def test_embed_and_gather_are_exact(ops, dtype, T, H, V):
+    table = rnd(V, H, dtype=dtype)
+    ids = torch.randint(0, V, (T,), dtype=torch.int32, device="cuda")
+    out = ops.embed(ids, table)
+    assert torch.equal(out, table[ids.long()])
+    rows = torch.randint(0, T, (5,), dtype=torch.int32, device="cuda")
+    assert torch.equal(ops.gather_rows(out, rows), out[rows.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H,eps", [(3, 80, 1e-5), (17, 1000, 1e-6), (5, 4096, 1e-6), (2, 12288, 1e-3)])
+def test_rmsnorm(ops, dtype, T, H, eps):
+    x = rnd(T, H, dtype=dtype, seed=1, scale=3.0)
+    w = (1 + 0.1 * torch.randn(H)).to(dtype).cuda()
+    y = ops.rmsnorm(x, w, eps)
+    xf = x.float()
+    ref = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    torch.testing.assert_close(y.float(), ref, **tol(dtype))
+    # with a residual: the carried sum is the rounded sum; the norm is of the unrounded one
+    res = rnd(T, H, dtype=dtype, seed=2, scale=3.0)
+    res_before = res.clone()
+    y2 = ops.rmsnorm(x, w, eps, residual=res)
+    s = x.float() + res_before.float()
+    assert torch.equal(res, s.to(dtype))
+    ref2 = s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    torch.testing.assert_close(y2.float(), ref2, **tol(dtype))
+
+
+def test_rmsnorm_float32_residual_with_bfloat16_rows(ops):
+    """The residual carried in float32: started from x exactly, then sums are not rounded."""
+    x = rnd(6, 200, dtype=torch.bfloat16, seed=1)
+    w = (1 + 0.1 * torch.randn(200)).bfloat16().cuda()
+    y, res = ops.rmsnorm(x, w, 1e-6, start_residual=True)
+    assert res.dtype == torch.float32 and torch.equal(res, x.float())
+    torch.testing.assert_close(y.float(), ops.rmsnorm(x, w, 1e-6).float(), rtol=0, atol=0)
+    x2 = rnd(6, 200, dtype=torch.bfloat16, seed=2)
+    y2 = ops.rmsnorm(x2, w, 1e-6, residual=res)
+    s = x.float() + x2.float()
+    assert torch.equal(res, s)
+    ref = s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + 1e-6) * w.float()
+    torch.testing.assert_close(y2.float(), ref, **tol(torch.bfloat16))
+
+
+def test_rmsnorm_float32_weight_with_bfloat16_rows(ops):
+    x = rnd(4, 96, dtype=torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(96)).cuda()
+    y = ops.rmsnorm(x, w, 1e-6)
+    xf = x.float()
+    ref = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16().float() * w
+    torch.testing.assert_close(y.float(), ref, **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(1, 112), (33, 1001), (64, 12288)])
+def test_silu_mul(ops, dtype, T, I):
+    gu = rnd(T, 2 * I, dtype=dtype, seed=3, scale=2.0)
+    out = ops.silu_mul(gu)
+    g, u = gu[:, :I].float(), gu[:, I:].float()
+    torch.testing.assert_close(out.float(), torch.nn.functional.silu(g) * u, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 301, 80), (7, 389, 96), (65, 130, 1000), (128, 256, 512), (3, 1000, 4104)])
+def test_linear(ops, dtype, M, N, K):
+    x = rnd(M, K, dtype=dtype, seed=4)
+    w = rnd(N, K, dtype=dtype, seed=5, scale=K ** -0.5)
+    b = rnd(N, dtype=dtype, seed=6)
+    ref = x.double() @ w.double().T
+    t = dict(rtol=1e-5, atol=2e-5) if dtype == torch.float32 else tol(dtype)
+    torch.testing.assert_close(ops.linear(x, w).double(), ref, **t)
+    torch.testing.assert_close(ops.linear(x, w, b).double(), ref + b.double(), **t)
+    if dtype == torch.bfloat16:
+        # float32 output from bfloat16 inputs (the logits): only the accumulation rounds
+        torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32).double(), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_linear_rows_do_not_depend_on_the_batch_in_float32(ops):
+    x = rnd(70, 200, seed=7)
+    w = rnd(150, 200, seed=8)
+    full = ops.linear(x, w)
+    for rows in ([0], [69], [3, 4, 5], list(range(64, 70))):
+        part = ops.linear(x[rows].contiguous(), w)
+        assert torch.equal(part, full[rows])
+
+
+def _rope_reference(x, positions, base, rot):
+    inv = 1.0 / (base ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
+    ang = positions.float()[:, None] * inv[None, :]
+    cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+    x1, x2 = x[..., :rot // 2], x[..., rot // 2:rot]
+    return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., rot:]), dim=-1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,rot,norm,bias", [
+    (4, 2, 16, 16, True, False), (6, 1, 32, 32, True, False), (5, 5, 48, 48, False, True),
+    (3, 3, 80, 40, True, False), (32, 8, 128, 128, True, False), (2, 1, 256, 0, False, False),
+])
+def test_qk_rope_write(ops, dtype, Hq, Hkv, D, rot, norm, bias):
+    from nanohybrid_vlm_amd.parts.positions import RotaryEmbedding
+    T, page, pages, eps, base = 23, 8, 9, 1e-5, 10000.0
+    width = (Hq + 2 * Hkv) * D
+    qkv = rnd(T, width, dtype=dtype, seed=9, scale=2.0)
+    b = rnd(width, dtype=dtype, seed=10) if bias else None
+    qw = (1 + 0.1 * torch.randn(D)).to(dtype).cuda() if norm else None
+    kw = (1 + 0.1 * torch.randn(D)).to(dtype).cuda() if norm else None
+    table = RotaryEmbedding(rot, 300, base).table.cuda() if rot else None
+    positions = torch.randint(0, 300, (T,), dtype=torch.int32, device="cuda")
+    slots = torch.randperm(page * pages)[:T].to(torch.int32).cuda()
+    slots[5] = -1                                     # a token that is not stored
+    k_cache = torch.zeros(pages, page, Hkv, D, dtype=dtype, device="cuda")
+    v_cache = torch.zeros_like(k_cache)
+    q = ops.qk_rope_write(qkv, b, qw, kw, eps, table, positions, slots, k_cache, v_cache, Hq, Hkv, D)
+
+    x = qkv.float()
+    if bias:
+        x = (x + b.float()).to(dtype).float()
+    qr = x[:, :Hq * D].reshape(T, Hq, D)
+    kr = x[:, Hq * D:(Hq + Hkv) * D].reshape(T, Hkv, D)
+    vr = x[:, (Hq + Hkv) * D:].reshape(T, Hkv, D)
+    if norm:
+        qr = qr * torch.rsqrt(qr.pow(2).mean(-1, keepdim=True) + eps) * qw.float()
+        kr = kr * torch.rsqrt(kr.pow(2).mean(-1, keepdim=True) + eps) * kw.float()
+    if rot:
+        qr = _rope_reference(qr.cpu(), positions.cpu(), base, rot).cuda()
+        kr = _rope_reference(kr.cpu(), positions.cpu(), base, rot).cuda()
+    t = tol(dtype) if dtype == torch.bfloat16 else dict(rtol=1e-5, atol=2e-5)
+    torch.testing.assert_close(q.float(), qr, **t)
+    stored = slots >= 0
+    kf, vf = k_cache.view(-1, Hkv, D), v_cache.view(-1, Hkv, D)
+    torch.testing.assert_close(kf[slots[stored].long()].float(), kr[stored], **t)
+    assert torch.equal(vf[slots[stored].long()], vr[stored].to(dtype))      # values are only moved
+    untouched = torch.ones(page * pages, dtype=torch.bool, device="cuda")
+    untouched[slots[stored].long()] = False
+    assert not kf[untouched].any() and not vf[untouched].any()
+
+
+def _paged_setup(dtype, lens, q_lens, Hq, Hkv, D, page, seed=0, scale=1.0):
+    """Requests with ``lens`` keys each whose last ``q_lens`` tokens are this step's queries; pages handed out
+    in a shuffled order. Returns the pieces for ops.paged_attention and the dense keys and values."""
+    from nanohybrid_vlm_amd.native.ops import AttentionBatch
+    g = torch.Generator().manual_seed(seed)
+    B = len(lens)
+    n_pages = sum(-(-n // page) for n in lens) + 3
+    order = torch.randperm(n_pages, generator=g).tolist()
+    k_cache = torch.full((n_pages, page, Hkv, D), float("nan"), dtype=dtype)
+    v_cache = torch.full((n_pages, page, Hkv, D), float("nan"), dtype=dtype)
+    width = max(-(-n // page) for n in lens)
+    bt = torch.full((B, width), -1, dtype=torch.int32)
+    ks, vs, qs, token_req, positions = [], [], [], [], []
+    for r, (n, nq) in enumerate(zip(lens, q_lens)):
+        k = (torch.randn(n, Hkv, D, generator=g) * scale).to(dtype)
+        v = torch.randn(n, Hkv, D, generator=g).to(dtype)
+        ks.append(k)
+        vs.append(v)
+        for lp in range(-(-n // page)):
+            pid = order.pop()
+            bt[r, lp] = pid
+            m = min(page, n - lp * page)
+            k_cache[pid, :m] = k[lp * page:lp * page + m]
+            v_cache[pid, :m] = v[lp * page:lp * page + m]
+        qs.append((torch.randn(nq, Hq, D, generator=g) * scale).to(dtype))
+        token_req += [r] * nq
+        positions += list(range(n - nq, n))
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    batch = AttentionBatch(num_tokens=sum(q_lens), num_requests=B,
+                           token_req=torch.tensor(token_req, dtype=torch.int32).cuda(),
+                           positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+                           cu_seqlens_q=cu.cuda(), context_lens=torch.tensor(lens, dtype=torch.int32).cuda(),
+                           max_q_len=max(q_lens), max_context_len=max(lens))
+    return torch.cat(qs).cuda(), k_cache.cuda(), v_cache.cuda(), batch, bt.cuda(), ks, vs, qs
+
+
+def _attention_reference(qs, ks, vs, lens, q_lens, scale, window):
+    outs = []
+    for q, k, v, n, nq in zip(qs, ks, vs, lens, q_lens):
+        Hq, Hkv = q.shape[1], k.shape[1]
+        kk = k.double().repeat_interleave(Hq // Hkv, dim=1)
+        vv = v.double().repeat_interleave(Hq // Hkv, dim=1)
+        s = torch.einsum("qhd,khd->hqk", q.double(), kk) * scale
+        qpos = torch.arange(n - nq, n)[:, None]
+        kpos = torch.arange(n)[None, :]
+        ok = kpos <= qpos
+        if window:
+            ok &= kpos > qpos - window
+        s = s.masked_fill(~ok[None], float("-inf"))
+        outs.append(torch.einsum("hqk,khd->qhd", torch.softmax(s, dim=-1), vv))
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [
+    (4, 2, 16, 4, None), (6, 1, 32, 8, None), (5, 5, 48, 7, None), (3, 1, 80, 16, 9),
+    (8, 2, 128, 64, None), (32, 8, 128, 256, None), (2, 2, 64, 5, 64), (7, 7, 112, 3, None),
+])
+def test_paged_attention(ops, dtype, Hq, Hkv, D, page, window):
+    # whole prompts, portions with earlier keys, single decoded tokens, a length of one, page edges
+    lens = [1, 64, 65, 300, 17, 128, 5, 257]
+    q_lens = [1, 64, 1, 43, 2, 1, 5, 1]
+    scale = D ** -0.5
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(dtype, lens, q_lens, Hq, Hkv, D, page, seed=11, scale=1.5)
+    out = ops.paged_attention(q, kc, vc, batch, bt, scale, window)
+    ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, window)
+    t = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else tol(dtype)
+    torch.testing.assert_close(out.double().cpu(), ref, **t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page", [8, 64, 256])
+def test_attention_finds_one_far_key(ops, dtype, page):
+    """One key is made to stand out (score far above the rest): the output must be that key's value,
+    wherever the key lies: first of the sequence, last of a page, first of a page, the query's own position."""
+    Hq, Hkv, D, n = 8, 2, 64, 700
+    for far in [0, page - 1, page, 2 * page - 1, n // 2, n - 2, n - 1]:
+        g = torch.Generator().manual_seed(far)
+        k = torch.randn(n, Hkv, D, generator=g) * 0.1
+        v = torch.randn(n, Hkv, D, generator=g)
+        q = torch.randn(1, Hq, D, generator=g) * 0.1
+        direction = torch.randn(D, generator=g)
+        direction = direction / direction.norm()
+        k[far] += 10.0 * direction
+        q[0] += 10.0 * direction                    # score of `far` is about 100 * D^-0.5 = 12.5 above the others
+        from nanohybrid_vlm_amd.native.ops import AttentionBatch
+        n_pages = -(-n // page)
+        perm = torch.randperm(n_pages, generator=g)
+        kc = torch.full((n_pages, page, Hkv, D), float("nan"))
+        vc = torch.full((n_pages, page, Hkv, D), float("nan"))
+        for lp in range(n_pages):
+            m = min(page, n - lp * page)
+            kc[perm[lp], :m] = k[lp * page:lp * page + m]
+            vc[perm[lp], :m] = v[lp * page:lp * page + m]
+        batch = AttentionBatch(1, 1, torch.zeros(1, dtype=torch.int32).cuda(),
+                               torch.tensor([n - 1], dtype=torch.int32).cuda(),
+                               torch.tensor([0, 1], dtype=torch.int32).cuda(),
+                               torch.tensor([n], dtype=torch.int32).cuda(), 1, n)
+        out = ops.paged_attention(q.to(dtype).cuda(), kc.to(dtype).cuda(), vc.to(dtype).cuda(), batch,
+                                  perm.to(torch.int32)[None].cuda(), D ** -0.5)
+        ref = _attention_reference([q.to(dtype)], [k.to(dtype)], [v.to(dtype)], [n], [1], D ** -0.5, None)
+        torch.testing.assert_close(out.double().cpu(), ref, **tol(dtype))
+        # and it is mostly that one value
+        kvh = torch.arange(Hq) // (Hq // Hkv)
+        assert (out.float().cpu()[0] - v[far, kvh]).abs().max() < 0.5, f"far key {far} not found"
+
+
+@pytest.mark.parametrize("V", [301, 389, 5000, 151936])
+def test_sampling(ops, V):
+    import plain_qwen3 as plain
+    g = torch.Generator().manual_seed(V)
+    n = 6
+    logits = (torch.randn(n, V, generator=g) * 3).cuda()
+    logits[0, 17] = logits[0, 200] = 50.0                # a tie: the first index wins
+    temps = torch.tensor([0.0, 0.0, 0.8, 1.0, 0.3, 2.5]).cuda()
+    keys = torch.tensor([0, 0, 1234567, -99, 2**62 + 5, 42], dtype=torch.int64).cuda()
+    tokens = ops.sample(logits, temps, keys).cpu()
+    assert tokens[0] == 17
+    assert tokens[1] == logits[1].argmax().item()
+    if V <= 5000:
+        mask = (1 << 64) - 1
+        for r in range(2, n):
+            key = int(keys[r]) & mask
+            # the noise of plain_qwen3.sample_noise for an already mixed key
+            noise = torch.tensor([-math.log(((_mix(key ^ i) >> 40) + 1) / 16777216.0) for i in range(V)])
+            assert tokens[r] == plain.sample_token(logits[r].cpu(), float(temps[r]), noise)
+
+
+def _mix(z):
+    mask = (1 << 64) - 1
+    z = (z + 0x9E3779B97F4A7C15) & mask
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+    return z ^ (z >> 31)
+
+
+def test_sampling_follows_the_distribution(ops):
+    """Empirical frequencies of 4000 draws against softmax(logits / T) (chi-square, fixed keys)."""
+    V, draws, temp = 12, 4000, 0.7
+    logits = torch.tensor([[2.0, 1.0, 0.5, 0.0, -0.5, -1.0, 1.5, 0.2, -2.0, 0.7, 0.1, -0.3]])
+    p = torch.softmax(logits[0] / temp, dim=0)
+    rows = logits.repeat(draws, 1).cuda()
+    keys = torch.arange(draws, dtype=torch.int64).cuda() * 7919 + 13
+    tokens = ops.sample(rows, torch.full((draws,), temp).cuda(), keys).cpu()
+    counts = torch.bincount(tokens.long(), minlength=V).float()
+    chi2 = ((counts - draws * p) ** 2 / (draws * p)).sum().item()
+    assert chi2 < 31.3, f"chi-square {chi2:.1f} with 11 degrees of freedom (0.999 quantile is 31.3)"
+
+
+def test_refusals(ops):
+    from nanohybrid_vlm_amd.native.ops import KernelError
+    x = rnd(2, 64)
+    with pytest.raises(KernelError, match="columns"):
+        ops.linear(x, rnd(8, 32))
+    with pytest.raises(KernelError, match="element type"):
+        ops.linear(x.half(), rnd(8, 64).half())
+    with pytest.raises(KernelError, match="limit"):
+        ops.rmsnorm(rnd(1, 20000), rnd(20000), 1e-6)
+    with pytest.raises(KernelError, match="contiguous"):
+        ops.rmsnorm(rnd(4, 128)[:, ::2], rnd(64), 1e-6)
+    with pytest.raises(KernelError, match="device"):
+        ops.rmsnorm(torch.zeros(2, 8), torch.ones(8), 1e-6)

@@ -1,0 +1,131 @@
+"""The same requests fed whole, with a decoded tail, in portions and mixed with
+others on few pages must give the plain implementation's logits at every position.
+
+Without a GPU the engine's logic runs on the CPU stand-in for the kernels
+(float32 only); with ``-m gpu`` it runs on the HIP kernels in float32 and bfloat16.
+"""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import replay_cases as rc
+from helpers import TOLERANCE, first_difference, max_abs_diff, sharpen
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _requests(vocab):
+    # lengths around page edges (pages of 8 and 64) and one long request
+    return {f"r{i}": rc.random_tokens(vocab, n, 100 + i) for i, n in enumerate([5, 64, 33, 65, 130, 17, 96, 1, 40])}
+
+
+def _plain_logits(folder, requests):
+    cfg, w = plain.read_model_folder(folder)
+    return {rid: plain.logits(cfg, w, toks) for rid, toks in requests.items()}
+
+
+def _check(got, want, tol, what):
+    for rid in want:
+        assert got[rid].shape == want[rid].shape, f"{what}: request {rid}: shape {got[rid].shape}"
+        d = max_abs_diff(got[rid], want[rid])
+        assert d <= tol, f"{what}: request {rid}: max diff {d:.3e} > {tol:.1e}; {first_difference(got[rid], want[rid], tol)}"
+
+
+def _run_all_modes(make_runner, folder, dtype):
+    cfg, _ = plain.read_model_folder(folder)
+    requests = _requests(cfg["vocab_size"])
+    want = _plain_logits(folder, requests)
+    tol = TOLERANCE[dtype]
+    results = {}
+    for mode, steps, page, pages in [
+        ("whole", rc.whole(requests), 8, 20),
+        ("tail", rc.tail_decoded(requests), 8, 20),
+        ("portions", rc.portions(requests), 8, 20),
+        # so few pages that every page is used again several times
+        ("mixed", rc.mixed(requests), 8, None),
+    ]:
+        if pages is None:
+            pages = rc.peak_tokens(steps, page) // page
+        runner = make_runner(folder, dtype, page, pages)
+        results[mode] = rc.run_in_process(runner, steps)
+        _check(results[mode], want, tol, f"{dtype} {mode}")
+        assert not runner.cache.requests, "every request was ended"
+        assert runner.cache.num_free_pages(0) == pages, "every page came back"
+    return results
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_replay_on_emulated_kernels(model_folders, emulated_kernels, name, tmp_path):
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+
+    def make(folder, dtype, page, pages):
+        return ModelRunner(folder, dtype=dtype, device="cpu", page_size=page, num_pages=pages, num_state_slots=4)
+
+    folder = model_folders[name]
+    if name != "C":
+        folder = sharpen(folder, str(tmp_path / "sharp"))
+    _run_all_modes(make, folder, "float32")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "A_sharp", "B_sharp"])
+def test_replay_on_gpu(model_folders, name, dtype, tmp_path):
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+
+    def make(folder, dtype, page, pages):
+        return ModelRunner(folder, dtype=dtype, device="cuda:0", page_size=page, num_pages=pages, num_state_slots=4)
+
+    folder = model_folders[name.split("_")[0]]
+    if name.endswith("_sharp"):
+        folder = sharpen(folder, str(tmp_path / "sharp"))
+    results = _run_all_modes(make, folder, dtype)
+    if dtype == "float32":
+        # in 32-bit the ways of cutting agree with each other far more closely than with the plain implementation
+        for mode in ("tail", "portions", "mixed"):
+            for rid in results["whole"]:
+                d = max_abs_diff(results[mode][rid], results["whole"][rid])
+                assert d <= 2e-6, f"float32 {mode} against whole: request {rid}: {d:.3e}"
+
+
+def _trace_run(folder, dtype, steps, out_dir, max_tokens, extra=()):
+    cmd = [sys.executable, os.path.join(REPO, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+           "--out", out_dir, "--max-tokens", str(max_tokens), *extra]
+    proc = subprocess.run(cmd, input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
+                          timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    done = [l for l in proc.stdout.splitlines() if l.startswith("done ")]
+    assert done == [f"done {s['step']}" for s in steps]
+    return proc
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_folders, dtype, tmp_path):
+    """The program itself, as a user starts it: mixed trace, pool made for the trace's peak, files compared."""
+    folder = model_folders["B"]
+    cfg, w = plain.read_model_folder(folder)
+    requests = {f"r{i}": rc.random_tokens(cfg["vocab_size"], n, 7 + i) for i, n in enumerate([70, 130, 9, 64, 65, 100])}
+    steps = rc.mixed(requests)
+    out_dir = str(tmp_path / "out")
+    _trace_run(folder, dtype, steps, out_dir, rc.peak_tokens(steps, 64))
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in requests.items()}
+    fed = {rid: 0 for rid in requests}
+    V = cfg["vocab_size"]
+    for st in steps:
+        data = np.fromfile(os.path.join(out_dir, f"{st['step']}.f32"), dtype="<f4").reshape(-1, V)
+        row = 0
+        for e in st["entries"]:
+            n = len(e["tokens"])
+            ref = want[e["id"]][fed[e["id"]]:fed[e["id"]] + n]
+            d = max_abs_diff(torch.from_numpy(data[row:row + n].copy()), ref)
+            assert d <= TOLERANCE[dtype], f"step {st['step']} request {e['id']}: {d:.3e}"
+            fed[e["id"]] += n
+            row += n
+        assert row == data.shape[0]
