@@ -29,6 +29,7 @@ class EngineConfig:
     num_state_slots: int = -1                   # -1: max_num_seqs
     dtype: str = "bfloat16"                     # "bfloat16" or "float32" (true 32-bit everywhere)
     seed: int = 0                               # default seed of temperature sampling
+    device: str = "cuda:0"                      # the one GPU
 
     def __post_init__(self):
         if self.dtype not in _DTYPES:

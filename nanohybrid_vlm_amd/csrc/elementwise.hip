@@ -2,20 +2,6 @@
 // the fused q/k-norm + rotation + cache-write kernel. All in two element types
 // (float, bfloat16); statistics, angles and sums are float.
 #include "nhv_common.h"
-#include <stdarg.h>
-#include <stdio.h>
-
-static thread_local char g_error[512] = "";
-
-int nhv_fail(const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_error, sizeof(g_error), fmt, ap);
-  va_end(ap);
-  return 1;
-}
-
-extern "C" const char* nhv_last_error() { return g_error; }
 
 // ---------------------------------------------------------------- embedding
 template <typename T>

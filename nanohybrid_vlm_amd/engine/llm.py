@@ -102,7 +102,7 @@ class LLM:
         if not os.path.isdir(model):
             raise FileNotFoundError(f"model folder '{model}' does not exist")
         self.runner = ModelRunner(
-            model, dtype=cfg.dtype, page_size=cfg.kvcache_block_size,
+            model, dtype=cfg.dtype, device=cfg.device, page_size=cfg.kvcache_block_size,
             num_pages=None if cfg.num_kvcache_blocks == -1 else cfg.num_kvcache_blocks,
             num_state_slots=cfg.max_num_seqs if cfg.num_state_slots == -1 else cfg.num_state_slots,
             gpu_memory_utilization=cfg.gpu_memory_utilization, max_num_batched_tokens=cfg.max_num_batched_tokens)
@@ -150,6 +150,7 @@ class LLM:
         t0 = perf_counter()
         plan = self.scheduler.schedule()
         seqs = plan.seqs
+        num_prefill_tokens, num_decode_tokens = plan.num_prefill_tokens, plan.num_decode_tokens
         entries, sampled_rows = [], []
         for seq in seqs:
             n = seq.num_scheduled_tokens
@@ -184,7 +185,7 @@ class LLM:
             self._completed_metrics.append(m)
             self._sequences.pop(s.seq_id, None)
             outputs.append((s.seq_id, s.completion_token_ids))
-        stats = StepStats(num_prefill_tokens=plan.num_prefill_tokens, num_decode_tokens=plan.num_decode_tokens,
+        stats = StepStats(num_prefill_tokens=num_prefill_tokens, num_decode_tokens=num_decode_tokens,
                           seconds=now - t0, num_preempted=len(plan.preempted_seq_ids))
         return outputs, stats
 

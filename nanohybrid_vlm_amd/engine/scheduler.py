@@ -160,7 +160,10 @@ class Scheduler:
                     return (num_active < self.max_num_seqs and self.cache.can_admit()
                             and self.cache.can_reserve(seq.seq_id, seq.num_tokens))
                 while reserve_prefill and not resources_available():
-                    victim = self._select_preemption_victim(scheduled_decode_ids)
+                    # requests that already have a place in this step stay: the decoding ones and (unlike
+                    # the reference, scheduler.py:674-719, which would push them out) the prompts just planned
+                    victim = self._select_preemption_victim(
+                        scheduled_decode_ids | {p.seq_id for p in plan.prefill_seqs})
                     if victim is None:
                         break
                     plan.preempted_seq_ids.append(victim.seq_id)

@@ -69,9 +69,8 @@ def _digest(sources: list[str], defines: list[str]) -> str:
 def _writable_dir() -> str:
     try:
         os.makedirs(LIB_DIR, exist_ok=True)
-        probe = os.path.join(LIB_DIR, f".probe{os.getpid()}")
-        with open(probe, "w"):
-            pass
+        fd, probe = tempfile.mkstemp(prefix=".probe", dir=LIB_DIR)
+        os.close(fd)
         os.remove(probe)
         return LIB_DIR
     except OSError:

@@ -16,7 +16,10 @@ import torch
 
 from . import library
 
-CORE_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip"]
+CORE_SOURCES = ["error.hip", "elementwise.hip", "gemm_generic.hip", "gemm_skinny_bf16.hip", "attention_generic.hip",
+                "sampling.hip"]
+ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip"]      # compiled once per head size
+ATTENTION_HEAD_DIMS_BUILT_AHEAD = [16, 32, 48, 64, 80, 96, 112, 128, 256]
 
 F32, BF16 = 0, 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -81,11 +84,22 @@ class NativeBackend:
             raise KernelError("no GPU is visible to torch; the HIP kernels are the only implementation")
         self.lib = library.load_library("nhv_core", CORE_SOURCES)
         self.lib.nhv_last_error.restype = ctypes.c_char_p
+        self._attention_libs: dict[int, ctypes.CDLL] = {}
 
-    def _call(self, fn_name: str, *args) -> None:
-        rc = getattr(self.lib, fn_name)(*args)
+    def _call(self, fn_name: str, *args, lib=None) -> None:
+        lib = lib or self.lib
+        rc = getattr(lib, fn_name)(*args)
         if rc != 0:
-            raise KernelError(self.lib.nhv_last_error().decode())
+            raise KernelError(lib.nhv_last_error().decode())
+
+    def attention_lib(self, head_dim: int) -> ctypes.CDLL:
+        """The bfloat16 attention kernels are compiled per head size, when a model first needs them."""
+        lib = self._attention_libs.get(head_dim)
+        if lib is None:
+            lib = library.load_library(f"nhv_attention_d{head_dim}", ATTENTION_SOURCES, [f"-DNHV_HEAD_DIM={head_dim}"])
+            lib.nhv_last_error.restype = ctypes.c_char_p
+            self._attention_libs[head_dim] = lib
+        return lib
 
     # -- each method launches one kernel; arguments were checked by the caller --
     def embed(self, ids, table, out):
@@ -117,13 +131,49 @@ class NativeBackend:
     def paged_attention(self, q, k_cache, v_cache, out, batch: AttentionBatch, block_tables, scale, window):
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
+        if (q.dtype == torch.bfloat16 and batch.max_q_len == 1 and D % 16 == 0 and D <= 512 and Hq // Hkv <= 16
+                and T <= 65535):
+            return self._decode_attention(q, k_cache, v_cache, out, batch, block_tables, scale, window)
         self._call("nhv_paged_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
                    _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables), block_tables.shape[1], T, Hq, Hkv,
                    D, page_size, ctypes.c_float(scale), window, dtype_code(q), _stream())
 
+    def _decode_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window):
+        """Single tokens in bfloat16: keys split over waves, then merged."""
+        T, Hq, D = q.shape
+        _, page_size, Hkv, _ = k_cache.shape
+        span = batch.max_context_len if not window else min(batch.max_context_len, window + 16)
+        # enough waves to fill the chip: about 2048 of them
+        want = max(1, T * Hkv * span // 2048)
+        split_len = 32
+        while split_len < want and split_len < 1024:
+            split_len *= 2
+        n_splits = -(-batch.max_context_len // split_len)
+        part_o = torch.empty((T, Hq, n_splits, D), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, Hq, n_splits, 2), dtype=torch.float32, device=q.device)
+        self._call("nhv_decode_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_o),
+                   _ptr(part_ml), _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables),
+                   block_tables.shape[1], T, Hq, Hkv, page_size, ctypes.c_float(scale), window, split_len, n_splits,
+                   _stream(), lib=self.attention_lib(D))
+
     def linear(self, x, w, bias, out):
         M, K = x.shape
         N = w.shape[0]
+        if x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
+            if M <= 64:
+                return self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
+                                  dtype_code(out), _stream())
+            if out.dtype == torch.bfloat16 and bias is None:
+                # many rows: the library's matrix product (the reference's linears are library calls too,
+                # nanovllm/layers/linear.py:88,192)
+                torch.mm(x, w.t(), out=out)
+                return None
+            if out.dtype == torch.float32:
+                for m0 in range(0, M, 64):          # float32 output of many rows (logits of a whole prompt)
+                    m1 = min(M, m0 + 64)
+                    self._call("nhv_gemm_skinny_bf16", _ptr(x[m0:m1]), _ptr(w), _ptr(bias), _ptr(out[m0:m1]),
+                               m1 - m0, N, K, dtype_code(out), _stream())
+                return None
         self._call("nhv_gemm_generic", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K, dtype_code(x),
                    dtype_code(out), _stream())
 

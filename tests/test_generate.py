@@ -1,0 +1,137 @@
+"""Generation through the entry point: greedy and seeded temperature sampling against
+the plain implementation, with prompts cut to a small token budget, with so few
+pages that requests are pushed out and computed again, and with late arrivals."""
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from conftest import TINY
+from nanohybrid_vlm_amd import LLM, SamplingParams
+from nanohybrid_vlm_amd.sampling.sampler import noise_key
+from replay_cases import random_tokens
+
+
+def _plain_generate(cfg, w, prompt, sp: SamplingParams, request: int, engine_seed: int, eos):
+    ids, out = list(prompt), []
+    for step in range(sp.max_tokens):
+        row = plain.logits(cfg, w, ids)[-1]
+        if sp.temperature == 0:
+            t = plain.sample_token(row, 0.0, None)
+        else:
+            seed = engine_seed if sp.seed is None else sp.seed
+            t = plain.sample_token(row, sp.temperature, plain.sample_noise(seed, request, step, row.numel()))
+        ids.append(t)
+        out.append(t)
+        if not sp.ignore_eos and t == eos:
+            break
+    return out
+
+
+def _workload(name):
+    cfg, _ = TINY[name]
+    lens = [5, 17, 33] if name == "A" else [1, 13, 40, 64]
+    return [random_tokens(cfg["vocab_size"], n, 50 + n) for n in lens]
+
+
+def _run(folder, device, dtype, name, **options):
+    cfg, w = plain.read_model_folder(folder)
+    prompts = _workload(name)
+    greedy = SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True)
+    llm = LLM(folder, device=device, dtype=dtype, **options)
+    outs = llm.generate(prompts, greedy, use_tqdm=False)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        assert o["text"] is None
+        assert o["token_ids"] == _plain_generate(cfg, w, p, greedy, i, 0, cfg.get("eos_token_id")), f"greedy, prompt {i}"
+    # temperature sampling with the engine's counter-based noise, one request with a seed of its own; ends at eos
+    params = [SamplingParams(temperature=0.8, max_tokens=12, seed=None if i % 2 else 1000 + i) for i in range(len(prompts))]
+    outs = llm.generate(prompts, params, use_tqdm=False)
+    for i, (p, sp, o) in enumerate(zip(prompts, params, outs)):
+        # request ids go on counting: the second batch has ids len(prompts)..
+        want = _plain_generate(cfg, w, p, sp, len(prompts) + i, llm.config.seed, llm.config.eos)
+        assert o["token_ids"] == want, f"temperature, prompt {i}"
+    metrics = llm.get_completed_request_metrics()
+    assert len(metrics) == 2 * len(prompts) and all(m.ttft_ms >= 0 and m.e2e_ms >= m.ttft_ms for m in metrics)
+    return llm
+
+
+@pytest.mark.parametrize("name,options", [
+    ("A", dict(kvcache_block_size=4, num_kvcache_blocks=64)),
+    ("B", dict(kvcache_block_size=8, num_kvcache_blocks=64, max_num_batched_tokens=7)),        # prompts in portions of 7
+    ("B", dict(kvcache_block_size=8, num_kvcache_blocks=13, max_num_batched_tokens=16, max_num_seqs=3)),  # pages run out
+])
+def test_generate_on_emulated_kernels(model_folders, emulated_kernels, name, options):
+    llm = _run(model_folders[name], "cpu", "float32", name, **options)
+    if options["num_kvcache_blocks"] == 13:
+        assert llm.scheduler.num_preemptions > 0, "the small cache was meant to force a request out"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,options", [
+    ("A", dict(kvcache_block_size=4, num_kvcache_blocks=64)),
+    ("B", dict(kvcache_block_size=8, num_kvcache_blocks=64, max_num_batched_tokens=7)),
+    ("B", dict(kvcache_block_size=8, num_kvcache_blocks=13, max_num_batched_tokens=16, max_num_seqs=3)),
+])
+def test_generate_float32_on_gpu(model_folders, name, options):
+    _run(model_folders[name], "cuda:0", "float32", name, **options)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_generate_bfloat16_on_gpu(model_folders, name):
+    """bfloat16 may choose the other of two nearly equal logits; every token must be one the plain
+    implementation also rates within the rounding of the best."""
+    folder = model_folders[name]
+    cfg, w = plain.read_model_folder(folder)
+    prompts = _workload(name)
+    llm = LLM(folder, dtype="bfloat16", kvcache_block_size=8, num_kvcache_blocks=64, max_num_batched_tokens=16)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
+    for p, o in zip(prompts, outs):
+        ids = list(p)
+        assert len(o["token_ids"]) == 8
+        for t in o["token_ids"]:
+            row = plain.logits(cfg, w, ids)[-1]
+            assert row[t] >= row.max() - 2e-2, "a token far from the best was chosen"
+            ids.append(t)
+
+
+def test_late_arrivals_and_step_by_hand(model_folders, emulated_kernels):
+    """Requests added while others decode (nanovllm's tests drive llm.step() the same way,
+    tests/5090-test-TP2/run_generation.py:62-134)."""
+    folder = model_folders["A"]
+    cfg, w = plain.read_model_folder(folder)
+    llm = LLM(folder, device="cpu", dtype="float32", kvcache_block_size=4, num_kvcache_blocks=64, max_num_batched_tokens=12)
+    sp = SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True)
+    first = [random_tokens(256, n, n) for n in (6, 9)]
+    late = [random_tokens(256, n, n) for n in (30, 21)]
+    ids = [llm.add_request(p, sp) for p in first]
+    done, mixed_steps = {}, 0
+    for _ in range(3):
+        out, _ = llm.step()
+    ids += [llm.add_request(p, sp) for p in late]
+    while not llm.is_finished():
+        out, stats = llm.step()
+        mixed_steps += bool(stats.num_decode_tokens and stats.num_prefill_tokens)
+        done.update(dict(out))
+    assert mixed_steps >= 2, "decoded tokens and prompt portions ran in one batch"
+    for i, p in zip(ids, first + late):
+        assert done[i] == plain.greedy_generate(cfg, w, p, 10)
+
+
+def test_entry_point_refusals(model_folders, emulated_kernels):
+    folder = model_folders["A"]
+    with pytest.raises(TypeError, match="unknown engine options"):
+        LLM(folder, device="cpu", tensor_parallel_size=2)
+    with pytest.raises(FileNotFoundError):
+        LLM(folder + "_nowhere", device="cpu")
+    llm = LLM(folder, device="cpu", dtype="float32", kvcache_block_size=4, num_kvcache_blocks=8, max_model_len=64)
+    assert llm.config.eos == 3 and llm.config.max_model_len == 64
+    for bad, err in [([], ValueError), ([1, -2], ValueError), ([1, True], TypeError), ("text", ValueError),
+                     ([1, 999], ValueError), ((1, 2), TypeError)]:
+        with pytest.raises(err):
+            llm.add_request(bad, SamplingParams())
+    with pytest.raises(ValueError, match="max_model_len"):
+        llm.add_request([1] * 60, SamplingParams(max_tokens=10))
+    with pytest.raises(ValueError):
+        SamplingParams(temperature=-1)
+    with pytest.raises(ValueError):
+        SamplingParams(temperature=float("nan"))

@@ -110,6 +110,20 @@ def test_linear(ops, dtype, M, N, K):
         torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32).double(), ref, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 1000, 12288), (16, 389, 96), (17, 301, 80), (33, 6144, 1024),
+                                   (48, 50, 2048), (64, 151936, 256), (64, 4096, 12288)])
+def test_skinny_linear_bfloat16(ops, M, N, K):
+    """Few rows in bfloat16 (a decoding step): own MFMA kernel, K split over waves."""
+    x = rnd(M, K, dtype=torch.bfloat16, seed=14)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=15, scale=K ** -0.5)
+    ref = x.double() @ w.double().T
+    torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32).double(), ref, rtol=1e-4, atol=2e-4)
+    torch.testing.assert_close(ops.linear(x, w).double(), ref, **tol(torch.bfloat16))
+    # a row's result does not depend on how many other rows there are (as long as the same kernel runs)
+    if M > 1:
+        assert torch.equal(ops.linear(x[:1].contiguous(), w, out_dtype=torch.float32), ops.linear(x, w, out_dtype=torch.float32)[:1])
+
+
 def test_linear_rows_do_not_depend_on_the_batch_in_float32(ops):
     x = rnd(70, 200, seed=7)
     w = rnd(150, 200, seed=8)
@@ -239,6 +253,28 @@ def test_paged_attention(ops, dtype, Hq, Hkv, D, page, window):
     ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, window)
     t = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else tol(dtype)
     torch.testing.assert_close(out.double().cpu(), ref, **t)
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [
+    (4, 2, 16, 4, None), (6, 1, 32, 8, None), (5, 5, 48, 7, None), (3, 1, 80, 16, 9), (8, 2, 128, 64, None),
+    (32, 8, 128, 256, None), (16, 1, 64, 5, 70), (7, 7, 112, 3, None), (2, 1, 256, 32, None), (12, 2, 96, 16, 300),
+])
+def test_decode_attention_bfloat16(ops, Hq, Hkv, D, page, window):
+    """Single tokens of several requests in bfloat16: the split-key kernel (lengths around the edges of
+    tiles of 16, of splits and of pages)."""
+    lens = [1, 15, 16, 17, 31, 32, 33, 64, 65, 300, 257, 1000, 1024, 1025]
+    q_lens = [1] * len(lens)
+    scale = D ** -0.5
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=21, scale=1.5)
+    out = ops.paged_attention(q, kc, vc, batch, bt, scale, window)
+    ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, window)
+    torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
+    # the same tokens one at a time (other split lengths are chosen then): same result up to rounding
+    one = ops.paged_attention(q[9:10].contiguous(), kc, vc,
+                              type(batch)(1, 1, torch.zeros(1, dtype=torch.int32).cuda(), batch.positions[9:10].contiguous(),
+                                          torch.tensor([0, 1], dtype=torch.int32).cuda(), batch.context_lens[9:10].contiguous(),
+                                          1, lens[9]), bt[9:10].contiguous(), scale, window)
+    torch.testing.assert_close(one.float(), out[9:10].float(), rtol=1e-2, atol=1e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

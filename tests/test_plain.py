@@ -1,0 +1,172 @@
+"""Pins of the plain implementation beside the reference's text: special cases that
+reduce to a library routine and invariants, each chosen so that a plausible mistake
+(a wrong sign or pairing, a swapped gate, a norm in the wrong place, a wrong group
+mapping) fails it. The reference holds no test vector for Qwen3 dense (its golden
+files are of another architecture), so whole-model parity is unpinned beyond these."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_qwen3 as plain
+from conftest import TINY_A, TINY_B
+
+
+def test_rms_norm_is_the_library_routine():
+    x = torch.randn(5, 96) * 3
+    w = 1 + 0.1 * torch.randn(96)
+    torch.testing.assert_close(plain.rms_norm(x, w, 1e-5), F.rms_norm(x, (96,), w, 1e-5))
+    # eps sits inside the root, added to the mean of squares: ||y||^2 = H ||x||^2 / (||x||^2 + H eps) for w = 1
+    eps = 0.5
+    y = plain.rms_norm(x, torch.ones(96), eps)
+    n2 = x.pow(2).sum(-1)
+    torch.testing.assert_close(y.pow(2).sum(-1), 96 * n2 / (n2 + 96 * eps))
+
+
+def test_add_rms_norm_norms_the_sum_and_carries_it():
+    x, r = torch.randn(4, 32), torch.randn(4, 32)
+    w = 1 + 0.1 * torch.randn(32)
+    y, s = plain.add_rms_norm(x, r, w, 1e-6)
+    assert torch.equal(s, x + r)
+    torch.testing.assert_close(y, plain.rms_norm(x + r, w, 1e-6))
+
+
+def test_rope_angles_against_float64():
+    pos = torch.arange(0, 300, 7)
+    for base, d in [(10000.0, 16), (1e6, 32), (50000.0, 48)]:
+        ang = plain.rope_angles(pos, d, base).double()
+        ref = pos.double()[:, None] * torch.tensor([base ** (-2 * j / d) for j in range(d // 2)], dtype=torch.float64)
+        torch.testing.assert_close(ang, ref, rtol=2e-6, atol=1e-4)
+
+
+def test_rope_pairs_first_half_with_second_half():
+    d = 16
+    x = torch.zeros(1, 1, d)
+    x[0, 0, 0] = 1.0                                       # only the first entry of the first half
+    y = plain.apply_rope(x, torch.tensor([3]), 10000.0)[0, 0]
+    # pair (0, d/2) turns by 3 * base^0 = 3 rad: (1, 0) -> (cos 3, sin 3); an interleaved pairing would fill y[1]
+    assert abs(y[0] - math.cos(3.0)) < 1e-6 and abs(y[d // 2] - math.sin(3.0)) < 1e-6
+    assert y[1] == 0 and y[d // 2 + 1] == 0
+    # the last pair turns slowest
+    x = torch.zeros(1, 1, d)
+    x[0, 0, d // 2 - 1] = 1.0
+    y = plain.apply_rope(x, torch.tensor([3]), 10000.0)[0, 0]
+    a = 3 * 10000.0 ** (-(d - 2) / d)
+    assert abs(y[d // 2 - 1] - math.cos(a)) < 1e-6 and abs(y[d - 1] - math.sin(a)) < 1e-6
+
+
+def test_rope_invariants():
+    q, k = torch.randn(9, 3, 32), torch.randn(9, 3, 32)
+    pos = torch.arange(9)
+    # position 0 is the identity
+    torch.testing.assert_close(plain.apply_rope(q[:1], pos[:1], 1e6), q[:1])
+    # lengths of pairs are kept
+    y = plain.apply_rope(q, pos + 11, 1e6)
+    torch.testing.assert_close(y[..., :16] ** 2 + y[..., 16:] ** 2, q[..., :16] ** 2 + q[..., 16:] ** 2)
+    # a product of a turned q and a turned k depends on the distance only
+    a = (plain.apply_rope(q, pos + 5, 1e4) * plain.apply_rope(k, pos + 2, 1e4)).sum(-1)
+    b = (plain.apply_rope(q, pos + 105, 1e4) * plain.apply_rope(k, pos + 102, 1e4)).sum(-1)
+    torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-4)
+    # and with the sign of the sine flipped it would not equal the complex product
+    z = torch.complex(q[..., :16], q[..., 16:]) * torch.polar(torch.ones(9, 1, 16), plain.rope_angles(pos + 11, 32, 1e6)[:, None, :])
+    torch.testing.assert_close(y, torch.cat((z.real, z.imag), -1))
+
+
+def test_attention_is_the_library_routine_for_full_heads():
+    T, H, D = 23, 4, 16
+    q, k, v = torch.randn(T, H, D), torch.randn(T, H, D), torch.randn(T, H, D)
+    ref = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True,
+                                         scale=D ** -0.5).transpose(0, 1)
+    torch.testing.assert_close(plain.causal_attention(q, k, v, D ** -0.5), ref, rtol=1e-5, atol=1e-5)
+
+
+def test_attention_groups_and_special_cases():
+    T, Hq, Hkv, D = 11, 6, 2, 8
+    q, k, v = torch.randn(T, Hq, D), torch.randn(T, Hkv, D), torch.randn(T, Hkv, D)
+    out = plain.causal_attention(q, k, v, 0.3)
+    # grouped heads equal full heads after repeating each kv head Hq/Hkv times in place (head h reads h // 3)
+    full = plain.causal_attention(q, k.repeat_interleave(3, dim=1), v.repeat_interleave(3, dim=1), 0.3)
+    torch.testing.assert_close(out, full)
+    assert not torch.allclose(out, plain.causal_attention(q, k.repeat(1, 3, 1), v.repeat(1, 3, 1), 0.3))
+    # the first position sees one key: its output is that value
+    torch.testing.assert_close(out[0], v[0].repeat_interleave(3, dim=0))
+    # a window of one sees only itself
+    torch.testing.assert_close(plain.causal_attention(q, k, v, 0.3, window=1), v.repeat_interleave(3, dim=1))
+    # a window as long as the sequence changes nothing
+    torch.testing.assert_close(plain.causal_attention(q, k, v, 0.3, window=T), out)
+
+
+def test_swiglu_gate_is_the_first_matrix():
+    x = torch.randn(5, 12)
+    wg, wu, wd = torch.randn(20, 12), torch.randn(20, 12), torch.randn(12, 20)
+    torch.testing.assert_close(plain.swiglu(x, wg, wu, wd), (F.silu(x @ wg.T) * (x @ wu.T)) @ wd.T)
+    assert not torch.allclose(plain.swiglu(x, wg, wu, wd), plain.swiglu(x, wu, wg, wd))
+
+
+def _random_weights(cfg, seed):
+    from nanohybrid_vlm_amd.weights.random_init import random_checkpoint_tensors
+    return {k: v.float() for k, v in random_checkpoint_tensors(cfg, seed).items()}
+
+
+@pytest.mark.parametrize("cfg,seed", [(TINY_A, 0), (TINY_B, 1)])
+def test_only_distances_between_positions_count(cfg, seed):
+    """Shifting all positions leaves the logits alone: positions enter through the rotation only."""
+    w = _random_weights(cfg, seed)
+    toks = torch.randint(0, cfg["vocab_size"], (19,)).tolist()
+    a = plain.logits(cfg, w, toks, first_position=0)
+    b = plain.logits(cfg, w, toks, first_position=37)
+    torch.testing.assert_close(a, b, rtol=1e-4, atol=2e-5)
+
+
+def test_causality_and_dead_layers():
+    cfg = TINY_A
+    w = _random_weights(cfg, 0)
+    toks = torch.randint(0, cfg["vocab_size"], (15,)).tolist()
+    full = plain.logits(cfg, w, toks)
+    # a position does not see later tokens
+    torch.testing.assert_close(plain.logits(cfg, w, toks[:9]), full[:9], rtol=1e-5, atol=1e-6)
+    # with the output projections of every layer at zero the layers add nothing:
+    # logits = norm(embedding) . embedding^T (tied), which fixes where the final norm sits
+    dead = dict(w)
+    for name in w:
+        if name.endswith("o_proj.weight") or name.endswith("down_proj.weight"):
+            dead[name] = torch.zeros_like(w[name])
+    e = w["model.embed_tokens.weight"]
+    ref = F.rms_norm(e[toks], (cfg["hidden_size"],), w["model.norm.weight"], cfg["rms_norm_eps"]) @ e.T
+    torch.testing.assert_close(plain.logits(cfg, dead, toks), ref, rtol=1e-5, atol=1e-6)
+
+
+def test_one_layer_one_head_by_hand():
+    """One layer, one head, one kv head: every step spelled out with library calls."""
+    cfg = dict(TINY_A, num_hidden_layers=1, num_attention_heads=1, num_key_value_heads=1, head_dim=16, hidden_size=16,
+               intermediate_size=24, vocab_size=50, tie_word_embeddings=False)
+    w = _random_weights(cfg, 3)
+    toks = [4, 9, 1, 30, 7]
+    eps = cfg["rms_norm_eps"]
+    p = "model.layers.0."
+    r = w["model.embed_tokens.weight"][toks]
+    x = F.rms_norm(r, (16,), w[p + "input_layernorm.weight"], eps)
+    q = F.rms_norm(x @ w[p + "self_attn.q_proj.weight"].T, (16,), w[p + "self_attn.q_norm.weight"], eps)
+    k = F.rms_norm(x @ w[p + "self_attn.k_proj.weight"].T, (16,), w[p + "self_attn.k_norm.weight"], eps)
+    v = x @ w[p + "self_attn.v_proj.weight"].T
+    pos = torch.arange(5)
+    ang = pos[:, None].float() * (10000.0 ** (-torch.arange(0, 16, 2).float() / 16))[None]
+    rot = lambda t: torch.cat((t[:, :8] * ang.cos() - t[:, 8:] * ang.sin(), t[:, 8:] * ang.cos() + t[:, :8] * ang.sin()), -1)
+    o = F.scaled_dot_product_attention(rot(q)[None], rot(k)[None], v[None], is_causal=True, scale=0.25)[0]
+    r = r + o @ w[p + "self_attn.o_proj.weight"].T
+    x = F.rms_norm(r, (16,), w[p + "post_attention_layernorm.weight"], eps)
+    r = r + (F.silu(x @ w[p + "mlp.gate_proj.weight"].T) * (x @ w[p + "mlp.up_proj.weight"].T)) @ w[p + "mlp.down_proj.weight"].T
+    ref = F.rms_norm(r, (16,), w["model.norm.weight"], eps) @ w["lm_head.weight"].T
+    torch.testing.assert_close(plain.logits(cfg, w, toks), ref, rtol=1e-5, atol=1e-6)
+
+
+def test_sampling_rule():
+    row = torch.tensor([0.1, 2.0, 2.0, -1.0])
+    assert plain.sample_token(row, 0.0, None) == 1                      # argmax, first of equals
+    noise = torch.tensor([1e-3, 1.0, 1.0, 1.0])                          # tiny noise on index 0 wins: p / noise
+    assert plain.sample_token(row, 1.0, noise) == 0
+    n = plain.sample_noise(5, 2, 3, 1000)
+    assert (n >= 0).all() and abs(n.mean().item() - 1.0) < 0.1            # Exp(1) has mean 1
+    assert torch.equal(n, plain.sample_noise(5, 2, 3, 1000))
+    assert not torch.equal(n, plain.sample_noise(5, 2, 4, 1000))

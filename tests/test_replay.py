@@ -37,10 +37,27 @@ def _check(got, want, tol, what):
         assert d <= tol, f"{what}: request {rid}: max diff {d:.3e} > {tol:.1e}; {first_difference(got[rid], want[rid], tol)}"
 
 
-def _run_all_modes(make_runner, folder, dtype):
+def _rounding_reference(folder, requests):
+    """bfloat16 with sharpened attention: rounding q and k to 8 bits moves scores of size 16 by up to 0.06
+    and the logits by several 1e-2, which would hide a lost key. There the reference is the CPU stand-in for
+    the kernels run in bfloat16 (same places of rounding, whole requests, its float32 run is itself checked
+    against the plain implementation), and the tolerance stays that of bfloat16."""
+    from emulated_kernels import EmulatedBackend
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    from nanohybrid_vlm_amd.native import ops
+    old = ops._backend
+    ops.set_backend(EmulatedBackend())
+    try:
+        runner = ModelRunner(folder, dtype="bfloat16", device="cpu", page_size=16, num_pages=16, num_state_slots=2)
+        return rc.run_in_process(runner, rc.whole(requests))
+    finally:
+        ops.set_backend(old)
+
+
+def _run_all_modes(make_runner, folder, dtype, rounding_reference=False):
     cfg, _ = plain.read_model_folder(folder)
     requests = _requests(cfg["vocab_size"])
-    want = _plain_logits(folder, requests)
+    want = _rounding_reference(folder, requests) if rounding_reference else _plain_logits(folder, requests)
     tol = TOLERANCE[dtype]
     results = {}
     for mode, steps, page, pages in [
@@ -85,7 +102,7 @@ def test_replay_on_gpu(model_folders, name, dtype, tmp_path):
     folder = model_folders[name.split("_")[0]]
     if name.endswith("_sharp"):
         folder = sharpen(folder, str(tmp_path / "sharp"))
-    results = _run_all_modes(make, folder, dtype)
+    results = _run_all_modes(make, folder, dtype, rounding_reference=(dtype == "bfloat16" and name.endswith("_sharp")))
     if dtype == "float32":
         # in 32-bit the ways of cutting agree with each other far more closely than with the plain implementation
         for mode in ("tail", "portions", "mixed"):
