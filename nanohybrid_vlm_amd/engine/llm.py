@@ -94,25 +94,30 @@ def _load_tokenizer(folder: str):
 
 
 class LLM:
-    def __init__(self, model: str, **kwargs):
+    def __init__(self, model: str, *, built_model=None, **kwargs):
+        """``model``: folder with config.json, model.safetensors (and tokenizer.json for text prompts).
+        ``built_model``: (architecture, typed configuration, model with weights bound) made elsewhere, e.g.
+        with random weights drawn on the device; ``model`` is then only a label."""
         unknown = set(kwargs) - EngineConfig.field_names()
         if unknown:
             raise TypeError(f"unknown engine options: {sorted(unknown)}; known: {sorted(EngineConfig.field_names())}")
         self.config = cfg = EngineConfig(model=model, **kwargs)
-        if not os.path.isdir(model):
+        if built_model is None and not os.path.isdir(model):
             raise FileNotFoundError(f"model folder '{model}' does not exist")
+        arch, typed, built = built_model if built_model is not None else (None, None, None)
         self.runner = ModelRunner(
             model, dtype=cfg.dtype, device=cfg.device, page_size=cfg.kvcache_block_size,
             num_pages=None if cfg.num_kvcache_blocks == -1 else cfg.num_kvcache_blocks,
             num_state_slots=cfg.max_num_seqs if cfg.num_state_slots == -1 else cfg.num_state_slots,
-            gpu_memory_utilization=cfg.gpu_memory_utilization, max_num_batched_tokens=cfg.max_num_batched_tokens)
+            gpu_memory_utilization=cfg.gpu_memory_utilization, max_num_batched_tokens=cfg.max_num_batched_tokens,
+            model=built, arch=arch, cfg=typed)
         model_cfg = self.runner.cfg
         cfg.num_kvcache_blocks = self.runner.num_pages
         # max_model_len is capped by the model's positions (nanovllm/config.py:420-423)
         cfg.max_model_len = min(cfg.max_model_len, model_cfg.max_position_embeddings)
         if cfg.eos == -1 and getattr(model_cfg, "eos_token_id", None) is not None:
             cfg.eos = model_cfg.eos_token_id
-        self.tokenizer = _load_tokenizer(model)
+        self.tokenizer = _load_tokenizer(model) if built_model is None else None
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.eos,
                                    cfg.max_model_len, cfg.scheduler_policy, cfg.max_prefill_wait_ms)
         self.sampler = Sampler(self.runner.vocab_size)
