@@ -59,6 +59,7 @@ def build_llm(args, max_seqs):
     llm = LLM(f"random {args.shape}", built_model=(arch, cfg, model), dtype=args.dtype,
               kvcache_block_size=args.block_size, num_kvcache_blocks=max_seqs * pages_per_seq + 1,
               max_num_seqs=max_seqs, max_num_batched_tokens=max(2048, max_seqs), max_model_len=args.context,
+              scheduler_policy="prefill_first",     # while prompts are fed nothing decodes, so all requests decode in step
               enforce_eager=args.eager)
     return llm, cfg, full_layers
 

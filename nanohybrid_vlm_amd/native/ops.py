@@ -18,7 +18,7 @@ from . import library
 
 CORE_SOURCES = ["error.hip", "elementwise.hip", "gemm_generic.hip", "gemm_skinny_bf16.hip", "attention_generic.hip",
                 "sampling.hip"]
-ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip"]      # compiled once per head size
+ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip", "attention_prefill_bf16.hip"]      # compiled once per head size
 ATTENTION_HEAD_DIMS_BUILT_AHEAD = [16, 32, 48, 64, 80, 96, 112, 128, 256]
 
 F32, BF16 = 0, 1
@@ -134,6 +134,12 @@ class NativeBackend:
         if (q.dtype == torch.bfloat16 and batch.max_q_len == 1 and D % 16 == 0 and D <= 512 and Hq // Hkv <= 16
                 and T <= 65535):
             return self._decode_attention(q, k_cache, v_cache, out, batch, block_tables, scale, window)
+        if q.dtype == torch.bfloat16 and D % 16 == 0 and D <= 256 and batch.num_requests <= 65535 and Hkv <= 65535:
+            # prompt portions (and whatever single tokens share their batch) on the matrix cores
+            return self._call("nhv_prefill_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
+                              _ptr(batch.cu_seqlens_q), _ptr(batch.context_lens), _ptr(block_tables),
+                              block_tables.shape[1], batch.num_requests, batch.max_q_len, Hq, Hkv, page_size,
+                              ctypes.c_float(scale), window, _stream(), lib=self.attention_lib(D))
         self._call("nhv_paged_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
                    _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables), block_tables.shape[1], T, Hq, Hkv,
                    D, page_size, ctypes.c_float(scale), window, dtype_code(q), _stream())

@@ -277,6 +277,22 @@ def test_decode_attention_bfloat16(ops, Hq, Hkv, D, page, window):
     torch.testing.assert_close(one.float(), out[9:10].float(), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [
+    (4, 1, 128, 256, None), (8, 2, 64, 16, None), (6, 1, 32, 8, 100), (3, 3, 48, 5, None), (16, 1, 16, 64, None),
+    (5, 1, 256, 32, None), (32, 8, 128, 64, 700),
+])
+def test_prefill_attention_bfloat16(ops, Hq, Hkv, D, page, window):
+    """Long portions with and without earlier keys in bfloat16: the matrix-core kernel (tiles of 64 keys and of
+    16 tokens; portions that end inside a tile; a single token beside them)."""
+    lens = [700, 300, 64, 1500, 17, 129]
+    q_lens = [300, 300, 1, 1025, 16, 65]
+    scale = D ** -0.5
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=31, scale=1.5)
+    out = ops.paged_attention(q, kc, vc, batch, bt, scale, window)
+    ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, window)
+    torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("page", [8, 64, 256])
 def test_attention_finds_one_far_key(ops, dtype, page):
@@ -309,6 +325,16 @@ def test_attention_finds_one_far_key(ops, dtype, page):
                                   perm.to(torch.int32)[None].cuda(), D ** -0.5)
         ref = _attention_reference([q.to(dtype)], [k.to(dtype)], [v.to(dtype)], [n], [1], D ** -0.5, None)
         torch.testing.assert_close(out.double().cpu(), ref, **tol(dtype))
+        if far < n - 1:
+            # the same query once more as the second-to-last token of a portion of two (the portion kernel)
+            q2 = torch.cat((q, q)).to(dtype).cuda()
+            batch2 = AttentionBatch(2, 1, torch.zeros(2, dtype=torch.int32).cuda(),
+                                    torch.tensor([n - 2, n - 1], dtype=torch.int32).cuda(),
+                                    torch.tensor([0, 2], dtype=torch.int32).cuda(),
+                                    torch.tensor([n], dtype=torch.int32).cuda(), 2, n)
+            out2 = ops.paged_attention(q2, kc.to(dtype).cuda(), vc.to(dtype).cuda(), batch2,
+                                       perm.to(torch.int32)[None].cuda(), D ** -0.5)
+            torch.testing.assert_close(out2[1:].double().cpu(), ref, **tol(dtype))
         # and it is mostly that one value
         kvh = torch.arange(Hq) // (Hq // Hkv)
         assert (out.float().cpu()[0] - v[far, kvh]).abs().max() < 0.5, f"far key {far} not found"
