@@ -47,7 +47,6 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
     int page_size, float scale, int window, int split_len, int n_splits) {
   __shared__ float p_s[16][17];          // [key][head]
   __shared__ float alpha_s[16];
-  __shared__ int slot_s[16];
   const int lane = threadIdx.x;
   const int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
   const int G = Hq / Hkv;
@@ -76,30 +75,46 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
   const int ksub = lane / LPK, chunk = lane % LPK;
   const bool chunk_live = chunk * 8 < D;
 
-  for (int kb = (first / 16) * 16; kb <= last; kb += 16) {
-    // ---- scores of 16 keys
-    const int key_a = kb + col;
-    const bool ok_a = key_a >= first && key_a <= last;
-    int slot_a = 0;
-    if (ok_a) slot_a = bt[key_a / page_size] * page_size + key_a % page_size;
-    if (grp == 0) slot_s[col] = ok_a ? slot_a : -1;
-    const bf16_t* krow = k_cache + ((size_t)slot_a * Hkv + kvh) * D;
-    floatx4 s4 = {0.f, 0.f, 0.f, 0.f};
+  // keys of one round, as the first product's operand: lane loads 8 entries of key kb + col
+  auto load_keys = [&](int kb, bf16x8* ka) {
+    const int key = kb + col;
+    const bool ok = key >= first && key <= last;
+    int slot = 0;
+    if (ok) slot = bt[key / page_size] * page_size + key % page_size;
+    const bf16_t* krow = k_cache + ((size_t)slot * Hkv + kvh) * D;
 #pragma unroll
     for (int s = 0; s < DSTEPS; ++s) {
       const int d = s * 32 + grp * 8;
-      const bf16x8 ka = (ok_a && d < D) ? load8(krow + d) : zero8();
-      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[s], s4, 0, 0, 0);
+      ka[s] = (ok && d < D) ? load8(krow + d) : zero8();
     }
-    __syncthreads();                     // slot_s written; p_s and alpha_s of the last round are read
-    // ---- values of this round (issued early, used after the softmax)
+  };
+
+  const int kb0 = (first / 16) * 16;
+  bf16x8 ka[DSTEPS];
+  load_keys(kb0, ka);
+  for (int kb = kb0; kb <= last; kb += 16) {
+    // ---- this round's values and the next round's keys are asked for before anything is computed
     bf16x8 vv[PASSES];
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
       const int kl = ps * KPP + ksub;
-      const int sl = kl < 16 ? slot_s[kl] : -1;
-      vv[ps] = (chunk_live && sl >= 0) ? load8(v_cache + ((size_t)sl * Hkv + kvh) * D + chunk * 8) : zero8();
+      const int key = kb + kl;
+      const bool ok = chunk_live && kl < 16 && key >= first && key <= last;
+      int slot = 0;
+      if (ok) slot = bt[key / page_size] * page_size + key % page_size;
+      vv[ps] = ok ? load8(v_cache + ((size_t)slot * Hkv + kvh) * D + chunk * 8) : zero8();
     }
+    bf16x8 kn[DSTEPS];
+    if (kb + 16 <= last) {
+      load_keys(kb + 16, kn);
+    } else {
+#pragma unroll
+      for (int s = 0; s < DSTEPS; ++s) kn[s] = zero8();
+    }
+    // ---- scores of 16 keys
+    floatx4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < DSTEPS; ++s) s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[s], qb[s], s4, 0, 0, 0);
     // ---- running softmax for head `col` over keys kb + 4 grp + j
     float sc[4];
     float m_tile = -INFINITY;
@@ -114,6 +129,7 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
     const float m_new = fmaxf(m_run, m_tile);          // finite: every round holds a visible key
     const float alpha = expf(m_run - m_new);
     float psum = 0.f;
+    __syncthreads();                                   // the last round's p_s and alpha_s have been read
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float p = expf(sc[j] - m_new);             // exp(-inf) = 0 for keys out of range
@@ -146,6 +162,8 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
         }
       }
     }
+#pragma unroll
+    for (int s = 0; s < DSTEPS; ++s) ka[s] = kn[s];
   }
   // ---- this split's result: sum over the lanes that hold other keys of the same chunk
 #pragma unroll
@@ -174,24 +192,29 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
   }
 }
 
-// Merges the splits of every (token, head) in rising order of the keys.
+// Merges the splits of every (token, head): one wave each. The weights exp(m_s - M) are found with the lanes
+// spread over the splits; the outputs with the lanes spread over the head, adding the splits in rising order.
 __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                           bf16_t* __restrict__ out, const int* __restrict__ positions,
                                                           int window, int split_len, int n_splits, int Hq) {
   const int item = blockIdx.x;               // t * Hq + h
+  const int lane = threadIdx.x;
   const int t = item / Hq;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int s0 = lo / split_len, s1 = pos / split_len;
   const float* ml = part_ml + (size_t)item * n_splits * 2;
   float m = -INFINITY;
-  for (int s = s0; s <= s1; ++s) m = fmaxf(m, ml[s * 2]);
+  for (int s = s0 + lane; s <= s1; s += 64) m = fmaxf(m, ml[s * 2]);
+  m = wave_max(m);
   float l = 0.f;
-  for (int s = s0; s <= s1; ++s) l += ml[s * 2 + 1] * expf(ml[s * 2] - m);
+  for (int s = s0 + lane; s <= s1; s += 64) l += ml[s * 2 + 1] * expf(ml[s * 2] - m);
+  l = wave_sum(l);
   const float inv = 1.0f / l;
-  for (int d = threadIdx.x; d < D; d += 64) {
+  const float* po = part_o + (size_t)item * n_splits * D;
+  for (int d = lane; d < D; d += 64) {
     float o = 0.f;
-    for (int s = s0; s <= s1; ++s) o += part_o[((size_t)item * n_splits + s) * D + d] * expf(ml[s * 2] - m);
+    for (int s = s0; s <= s1; ++s) o += po[(size_t)s * D + d] * expf(ml[s * 2] - m);
     out[(size_t)item * D + d] = (bf16_t)(o * inv);
   }
 }

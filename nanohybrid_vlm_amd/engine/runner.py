@@ -45,7 +45,8 @@ class StepEntry:
 class ModelRunner:
     def __init__(self, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 256,
                  num_pages: int | None = None, num_state_slots: int = 512, gpu_memory_utilization: float = 0.9,
-                 max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None):
+                 max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None, use_graphs: bool = False,
+                 max_model_len: int | None = None, max_graph_batch: int = 64):
         """``model``/``arch``/``cfg`` may be given ready-made (weights already bound)
         instead of being read from ``model_dir``."""
         if dtype not in _TORCH_DTYPES:
@@ -66,6 +67,12 @@ class ModelRunner:
         self._make_cache(page_size, num_pages, num_state_slots, gpu_memory_utilization, max_num_batched_tokens)
         self._pinned = None
         self._pinned_free = None
+        # decode-only steps replay a HIP graph per batch-size bucket (the reference captures CUDA graphs for
+        # the same batch sizes, nanovllm/engine/model_runner.py:2559-2594)
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
+        self.max_model_len = min(max_model_len or self.max_position, self.max_position)
+        self.max_graph_batch = max_graph_batch
+        self._graphs: dict[int, dict] = {}
 
     # ------------------------------------------------------------------ cache
     def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens):
@@ -163,8 +170,11 @@ class ModelRunner:
             offset += n
         return out
 
-    def build_context(self, entries: list[StepEntry]) -> tuple[StepContext, list[int]]:
-        """Reserves pages and lays out the batch. Returns the context and every request's new length."""
+    def _layout(self, entries: list[StepEntry], pad_to: int | None = None, table_width: int | None = None):
+        """Reserves pages and lays the batch out as int32 arrays on the host.
+        ``pad_to``: number of requests the arrays are made for (a graph's bucket; only for
+        single-token entries): the padding rows store nothing and their results are dropped.
+        ``table_width``: fixed width of the block tables."""
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
@@ -189,35 +199,39 @@ class ModelRunner:
             new_lens.append(new_len)
 
         B = len(entries)
-        q_lens = np.array([len(e.tokens) for e in entries], dtype=np.int32)
+        pad = 0 if pad_to is None else pad_to - B
+        q_lens = np.array([len(e.tokens) for e in entries] + [1] * pad, dtype=np.int32)
         T = int(q_lens.sum())
-        cu = np.zeros(B + 1, dtype=np.int32)
+        cu = np.zeros(B + pad + 1, dtype=np.int32)
         np.cumsum(q_lens, out=cu[1:])
-        input_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        input_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries] + [np.zeros(pad, np.int64)])
         if input_ids.min() < 0 or input_ids.max() >= self.vocab_size:
             bad = int(input_ids[(input_ids < 0) | (input_ids >= self.vocab_size)][0])
             raise ValueError(f"token id {bad} is outside the vocabulary of {self.vocab_size}")
         input_ids = input_ids.astype(np.int32)
-        token_req = np.repeat(np.arange(B, dtype=np.int32), q_lens)
+        token_req = np.repeat(np.arange(B + pad, dtype=np.int32), q_lens)
         positions = (np.arange(T, dtype=np.int32) - np.repeat(cu[:-1], q_lens)
-                     + np.repeat(np.array(starts, dtype=np.int32), q_lens))
-        context_lens = np.array(new_lens, dtype=np.int32)
-        state_slots = np.array([cache.state_slot(e.request_id) for e in entries], dtype=np.int32)
+                     + np.repeat(np.array(starts + [0] * pad, dtype=np.int32), q_lens))
+        context_lens = np.array(new_lens + [1] * pad, dtype=np.int32)
+        state_slots = np.array([cache.state_slot(e.request_id) for e in entries] + [0] * pad, dtype=np.int32)
         rows = []
         for i, e in enumerate(entries):
             for w in e.want:
                 if not 0 <= w < len(e.tokens):
                     raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
                 rows.append(int(cu[i]) + w)
-        logit_rows = np.array(rows, dtype=np.int32)
 
-        arrays = [input_ids, positions, token_req, cu, context_lens, state_slots, logit_rows]
+        arrays = [input_ids, positions, token_req, cu, context_lens, state_slots]
         for gi, g in enumerate(cache.groups):
             tables = [cache.block_table(e.request_id, gi) for e in entries]
-            width = max(1, max(len(t) for t in tables))
-            bt = np.full((B, width), NO_PAGE, dtype=np.int32)
-            slot_mapping = np.empty(T, dtype=np.int32)
+            width = table_width or max(1, max(len(t) for t in tables))
+            # padding rows point at page 0 (a place that exists) and store nothing (slot -1)
+            bt = np.full((B + pad, width), NO_PAGE, dtype=np.int32)
+            bt[B:, 0] = 0
+            slot_mapping = np.full(T, -1, dtype=np.int32)
             for i, t in enumerate(tables):
+                if len(t) > width:
+                    raise ValueError(f"request {entries[i].request_id!r} holds {len(t)} pages; the tables have {width}")
                 ta = np.asarray(t, dtype=np.int32)
                 bt[i, :len(t)] = ta
                 p = positions[cu[i]:cu[i + 1]]
@@ -226,29 +240,112 @@ class ModelRunner:
                     raise RuntimeError(f"request {entries[i].request_id!r}: a new token falls on a page that was given back")
                 slot_mapping[cu[i]:cu[i + 1]] = pages * g.page_size + p % g.page_size
             arrays += [slot_mapping, bt]
-        dev = self._stage(arrays)
-        d_ids, d_pos, d_req, d_cu, d_ctx, d_slots, d_rows = dev[:7]
-        groups = [GroupTables(slot_mapping=dev[7 + 2 * gi], block_tables=dev[8 + 2 * gi])
-                  for gi in range(len(cache.groups))]
-        attention = AttentionBatch(num_tokens=T, num_requests=B, token_req=d_req, positions=d_pos, cu_seqlens_q=d_cu,
-                                   context_lens=d_ctx, max_q_len=int(q_lens.max()), max_context_len=int(max(new_lens)))
-        ctx = StepContext(num_tokens=T, num_requests=B, input_ids=d_ids, positions=d_pos, attention=attention,
-                          groups=groups, state_slots=d_slots, logit_rows=d_rows if len(rows) else None,
-                          num_logit_rows=len(rows),
-                          host={"starts": starts, "new_lens": new_lens, "q_lens": q_lens.tolist(),
-                                "state_slots": state_slots.tolist()})
-        return ctx, new_lens
+        meta = {"B": B + pad, "T": T, "rows": rows, "starts": starts, "new_lens": new_lens,
+                "q_lens": q_lens.tolist(), "state_slots": state_slots.tolist(),
+                "max_q_len": int(q_lens.max()), "max_context_len": int(max(new_lens))}
+        return arrays, meta
+
+    def _context(self, dev: list[torch.Tensor], meta: dict, logit_rows: torch.Tensor | None, num_logit_rows: int,
+                 max_context_len: int) -> StepContext:
+        d_ids, d_pos, d_req, d_cu, d_ctx, d_slots = dev[:6]
+        groups = [GroupTables(slot_mapping=dev[6 + 2 * gi], block_tables=dev[7 + 2 * gi])
+                  for gi in range(len(self.cache.groups))]
+        attention = AttentionBatch(num_tokens=meta["T"], num_requests=meta["B"], token_req=d_req, positions=d_pos,
+                                   cu_seqlens_q=d_cu, context_lens=d_ctx, max_q_len=meta["max_q_len"],
+                                   max_context_len=max_context_len)
+        return StepContext(num_tokens=meta["T"], num_requests=meta["B"], input_ids=d_ids, positions=d_pos,
+                           attention=attention, groups=groups, state_slots=d_slots, logit_rows=logit_rows,
+                           num_logit_rows=num_logit_rows,
+                           host={k: meta[k] for k in ("starts", "new_lens", "q_lens", "state_slots")})
+
+    def build_context(self, entries: list[StepEntry]) -> tuple[StepContext, list[int]]:
+        """Reserves pages, lays out the batch and copies it to the device. Returns the context and every
+        request's new length."""
+        arrays, meta = self._layout(entries)
+        rows = np.array(meta["rows"], dtype=np.int32)
+        dev = self._stage(arrays + [rows])
+        ctx = self._context(dev[:-1], meta, dev[-1] if len(rows) else None, len(rows), meta["max_context_len"])
+        return ctx, meta["new_lens"]
 
     @torch.no_grad()
     def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
         """Runs the batch and returns float32 logits [wanted, vocab] in the order of the
         entries and of each entry's ``want`` (None if nothing is wanted)."""
+        if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)
+                and not self.state_pools):
+            return self._graph_step(entries)
         ctx, new_lens = self.build_context(entries)
         hidden = self.model.forward(ctx)
         logits = self.model.logits(hidden) if hidden is not None else None
         for e, n in zip(entries, new_lens):
             self.cache.commit(e.request_id, n)
         return logits
+
+    # ------------------------------------------------------------------ decode steps as HIP graphs
+    def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+        """A step of single tokens: the batch is padded to a bucket, written into the bucket's fixed index
+        buffer, and the bucket's graph (embedding to logits of every row) is replayed."""
+        bucket = 1
+        while bucket < len(entries):
+            bucket *= 2
+        width = -(-self.max_model_len // self.page_size)
+        arrays, meta = self._layout(entries, pad_to=bucket, table_width=width)
+        if meta["max_context_len"] > width * self.page_size:
+            raise ValueError(f"a request of {meta['max_context_len']} tokens exceeds max_model_len {self.max_model_len}")
+        g = self._graphs.get(bucket)
+        if g is None:
+            g = self._graphs[bucket] = self._capture(bucket, arrays, meta, width)
+        sizes = [a.size for a in arrays]
+        total = sum(sizes)
+        if self._pinned is None or self._pinned.numel() < total:
+            self._pinned = torch.empty(max(total, 4096) * 2, dtype=torch.int32, pin_memory=True)
+            self._pinned_free = None
+        if self._pinned_free is not None:
+            self._pinned_free.synchronize()
+        flat = self._pinned[:total].numpy()
+        offset = 0
+        for a, n in zip(arrays, sizes):
+            flat[offset:offset + n] = a.reshape(-1)
+            offset += n
+        g["index"].copy_(self._pinned[:total], non_blocking=True)
+        self._pinned_free = torch.cuda.Event()
+        self._pinned_free.record()
+        g["graph"].replay()
+        for e, n in zip(entries, meta["new_lens"]):
+            self.cache.commit(e.request_id, n)
+        rows = meta["rows"]
+        if not rows:
+            return None
+        if rows == list(range(len(entries))):
+            return g["logits"][:len(entries)].clone()
+        return g["logits"][torch.tensor(rows, device=self.device)]
+
+    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int) -> dict:
+        """Runs the bucket's step once eagerly on its fixed buffers (so that every kernel library is loaded
+        and the allocator is warm), then records it."""
+        from ..native import ops
+        sizes = [a.size for a in arrays]
+        index = torch.zeros(sum(sizes), dtype=torch.int32, device=self.device)
+        host = torch.from_numpy(np.concatenate([a.reshape(-1) for a in arrays]))
+        index.copy_(host)
+        dev, offset = [], 0
+        for a, n in zip(arrays, sizes):
+            dev.append(index[offset:offset + n].view(a.shape))
+            offset += n
+        all_rows = torch.arange(bucket, dtype=torch.int32, device=self.device)
+        ctx = self._context(dev, meta, all_rows, bucket, max_context_len=width * self.page_size)
+        backend = ops.backend()
+        old = getattr(backend, "own_kernels_only", False)
+        backend.own_kernels_only = True                     # nothing of a library is recorded into the graph
+        try:
+            self.model.logits(self.model.forward(ctx))       # warm-up; it writes the same cache slots as the replay will
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.model.logits(self.model.forward(ctx))
+        finally:
+            backend.own_kernels_only = old
+        return {"graph": graph, "index": index, "logits": logits, "ctx": ctx}
 
     def finish(self, request_id) -> None:
         """The request is over: its pages and its state slot are given back."""

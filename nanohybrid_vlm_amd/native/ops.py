@@ -78,6 +78,7 @@ class NativeBackend:
 
     name = "hip"
     device_type = "cuda"
+    own_kernels_only = False      # True while a HIP graph is recorded: no library call goes into a graph
 
     def __init__(self):
         if not torch.cuda.is_available():
@@ -149,9 +150,9 @@ class NativeBackend:
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
         span = batch.max_context_len if not window else min(batch.max_context_len, window + 16)
-        # enough waves to fill the chip: about 2048 of them
-        want = max(1, T * Hkv * span // 2048)
-        split_len = 32
+        # enough waves to fill the chip (about 1024 of them), each with enough keys to be worth its start
+        want = max(1, T * Hkv * span // 1024)
+        split_len = 64
         while split_len < want and split_len < 1024:
             split_len *= 2
         n_splits = -(-batch.max_context_len // split_len)
@@ -166,16 +167,16 @@ class NativeBackend:
         M, K = x.shape
         N = w.shape[0]
         if x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
-            if M <= 64:
+            if M <= 16 or (M <= 64 and self.own_kernels_only):
                 return self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
                                   dtype_code(out), _stream())
-            if out.dtype == torch.bfloat16 and bias is None:
+            if out.dtype == torch.bfloat16 and bias is None and not self.own_kernels_only:
                 # many rows: the library's matrix product (the reference's linears are library calls too,
                 # nanovllm/layers/linear.py:88,192)
                 torch.mm(x, w.t(), out=out)
                 return None
             if out.dtype == torch.float32:
-                for m0 in range(0, M, 64):          # float32 output of many rows (logits of a whole prompt)
+                for m0 in range(0, M, 64):          # float32 output (logits), or more rows than a graph may hold in one call
                     m1 = min(M, m0 + 64)
                     self._call("nhv_gemm_skinny_bf16", _ptr(x[m0:m1]), _ptr(w), _ptr(bias), _ptr(out[m0:m1]),
                                m1 - m0, N, K, dtype_code(out), _stream())

@@ -91,13 +91,17 @@ def test_replay_on_emulated_kernels(model_folders, emulated_kernels, name, tmp_p
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C", "A_sharp", "B_sharp"])
-def test_replay_on_gpu(model_folders, name, dtype, tmp_path):
+def test_replay_on_gpu(model_folders, name, dtype, graphs, tmp_path):
+    """With ``graphs`` every step of single tokens replays a recorded HIP graph (one per batch size), between
+    eager steps of prompt portions: each replay is compared with the plain implementation."""
     from nanohybrid_vlm_amd.engine.runner import ModelRunner
 
     def make(folder, dtype, page, pages):
-        return ModelRunner(folder, dtype=dtype, device="cuda:0", page_size=page, num_pages=pages, num_state_slots=4)
+        return ModelRunner(folder, dtype=dtype, device="cuda:0", page_size=page, num_pages=pages, num_state_slots=4,
+                           use_graphs=graphs, max_model_len=160)
 
     folder = model_folders[name.split("_")[0]]
     if name.endswith("_sharp"):
