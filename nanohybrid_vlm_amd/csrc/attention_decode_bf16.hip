@@ -193,7 +193,13 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
 }
 
 // Merges the splits of every (token, head): one wave each. The weights exp(m_s - M) are found with the lanes
-// spread over the splits; the outputs with the lanes spread over the head, adding the splits in rising order.
+// spread over the splits. For the outputs a lane owns four consecutive entries of the head and every
+// (64 / lanes per row)-th split, with several loads in flight; the lanes' sums are then added across.
+constexpr int MQ = D / 4;                                   // float4 pieces of a row
+constexpr int MLPR = MQ <= 4 ? 4 : MQ <= 8 ? 8 : MQ <= 16 ? 16 : MQ <= 32 ? 32 : 64;   // lanes per row
+constexpr int MROWS = 64 / MLPR;                            // splits worked on side by side
+constexpr int MPIECES = (MQ + MLPR - 1) / MLPR;             // pieces per lane (more than 1 for heads above 256)
+
 __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                           bf16_t* __restrict__ out, const int* __restrict__ positions,
                                                           int window, int split_len, int n_splits, int Hq) {
@@ -212,10 +218,40 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
   l = wave_sum(l);
   const float inv = 1.0f / l;
   const float* po = part_o + (size_t)item * n_splits * D;
-  for (int d = lane; d < D; d += 64) {
-    float o = 0.f;
-    for (int s = s0; s <= s1; ++s) o += po[(size_t)s * D + d] * expf(ml[s * 2] - m);
-    out[(size_t)item * D + d] = (bf16_t)(o * inv);
+  const int sub = lane / MLPR, piece = lane % MLPR;
+  float4 acc[MPIECES];
+#pragma unroll
+  for (int i = 0; i < MPIECES; ++i) acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+  for (int s = s0 + sub; s <= s1; s += MROWS) {
+    const float wgt = expf(ml[s * 2] - m);
+#pragma unroll
+    for (int i = 0; i < MPIECES; ++i) {
+      const int qd = piece + i * MLPR;
+      if (qd < MQ) {
+        const float4 v = *reinterpret_cast<const float4*>(po + (size_t)s * D + qd * 4);
+        acc[i].x += v.x * wgt; acc[i].y += v.y * wgt; acc[i].z += v.z * wgt; acc[i].w += v.w * wgt;
+      }
+    }
+  }
+#pragma unroll
+  for (int off = MLPR; off < 64; off <<= 1) {
+#pragma unroll
+    for (int i = 0; i < MPIECES; ++i) {
+      acc[i].x += __shfl_xor(acc[i].x, off, 64); acc[i].y += __shfl_xor(acc[i].y, off, 64);
+      acc[i].z += __shfl_xor(acc[i].z, off, 64); acc[i].w += __shfl_xor(acc[i].w, off, 64);
+    }
+  }
+  if (sub == 0) {
+#pragma unroll
+    for (int i = 0; i < MPIECES; ++i) {
+      const int qd = piece + i * MLPR;
+      if (qd < MQ) {
+        bf16_t* o = out + (size_t)item * D + qd * 4;
+        o[0] = (bf16_t)(acc[i].x * inv); o[1] = (bf16_t)(acc[i].y * inv);
+        o[2] = (bf16_t)(acc[i].z * inv); o[3] = (bf16_t)(acc[i].w * inv);
+      }
+    }
   }
 }
 

@@ -57,6 +57,90 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, R* __restrict__ residual
   }
 }
 
+// The same for widths that are a multiple of 8: every thread owns up to MAXC pieces of 8 consecutive entries,
+// asks for all of them (rows, residual and weight) before it uses any, and keeps the sums in registers.
+template <typename V>
+__device__ __forceinline__ void load8f(const V* p, float* out) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = to_f32(p[e]);
+}
+template <>
+__device__ __forceinline__ void load8f<bf16_t>(const bf16_t* p, float* out) {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 v8;
+  const v8 v = *reinterpret_cast<const v8*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = (float)v[e];
+}
+template <>
+__device__ __forceinline__ void load8f<float>(const float* p, float* out) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w; out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+}
+template <typename V>
+__device__ __forceinline__ void store8f(V* p, const float* in) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) p[e] = from_f32<V>(in[e]);
+}
+template <>
+__device__ __forceinline__ void store8f<bf16_t>(bf16_t* p, const float* in) {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 v8;
+  v8 v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (__bf16)in[e];
+  *reinterpret_cast<v8*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void store8f<float>(float* p, const float* in) {
+  *reinterpret_cast<float4*>(p) = make_float4(in[0], in[1], in[2], in[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(in[4], in[5], in[6], in[7]);
+}
+
+template <typename T, typename W, typename R, int MAXC>
+__global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(const T* __restrict__ x, R* __restrict__ residual, int residual_mode,
+                                                           const W* __restrict__ w, T* __restrict__ y, int H, float eps) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * H;
+  const int nch = H / 8;
+  float v[MAXC][8], wv[MAXC][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ch = threadIdx.x + c * blockDim.x;
+    if (ch < nch) {
+      load8f<T>(x + base + ch * 8, v[c]);
+      load8f<W>(w + ch * 8, wv[c]);
+      if (residual_mode == 1) {
+        float r8[8];
+        load8f<R>(residual + base + ch * 8, r8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[c][e] += r8[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[c][e] = 0.f;
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ch = threadIdx.x + c * blockDim.x;
+    if (ch < nch && residual_mode != 0) store8f<R>(residual + base + ch * 8, v[c]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[c][e] * v[c][e];
+  }
+  const float total = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(total / (float)H + eps);
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ch = threadIdx.x + c * blockDim.x;
+    if (ch < nch) {
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = to_f32(from_f32<T>(v[c][e] * r)) * wv[c][e];
+      store8f<T>(y + base + ch * 8, o);
+    }
+  }
+}
+
 extern "C" int nhv_rmsnorm(const void* x, void* residual, int residual_mode, int residual_dtype, const void* w, void* y,
                            int T, int H, float eps, int dtype, int w_dtype, void* stream) {
   NHV_REQUIRE(T > 0 && H > 0, "rmsnorm: bad sizes T=%d H=%d", T, H);
@@ -64,11 +148,27 @@ extern "C" int nhv_rmsnorm(const void* x, void* residual, int residual_mode, int
   NHV_REQUIRE((residual_mode == 0) == (residual == nullptr), "rmsnorm: residual and its mode do not agree");
   const size_t lds = ((size_t)H + 16) * sizeof(float);
   NHV_REQUIRE(lds <= 64 * 1024, "rmsnorm: width %d is beyond this kernel's limit of %d", H, (64 * 1024) / 4 - 16);
-  const int threads = H >= 1024 ? 256 : 64;
   hipStream_t s = (hipStream_t)stream;
   if (residual_mode == 0) residual_dtype = NHV_F32;
-#define LAUNCH(TT, WW, RR) \
-  hipLaunchKernelGGL((rmsnorm_kernel<TT, WW, RR>), dim3(T), dim3(threads), lds, s, (const TT*)x, (RR*)residual, residual_mode, (const WW*)w, (TT*)y, H, eps)
+  // widths that are a multiple of 8 (with rows that then start on 16-byte borders) take the vector kernel
+  const bool vec = H % 8 == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
+                   ((uintptr_t)residual % 16 == 0);
+  const int nch = H / 8;
+  const int vthreads = nch <= 1024 ? ((nch + 63) / 64) * 64 : 1024;
+  const int maxc = (nch + vthreads - 1) / vthreads;       // 1 or 2: H <= 16368
+  const int threads = H >= 1024 ? 256 : 64;
+#define LAUNCH(TT, WW, RR)                                                                                              \
+  do {                                                                                                                  \
+    if (vec && maxc == 1)                                                                                               \
+      hipLaunchKernelGGL((rmsnorm_vec_kernel<TT, WW, RR, 1>), dim3(T), dim3(vthreads), 0, s, (const TT*)x, (RR*)residual, \
+                         residual_mode, (const WW*)w, (TT*)y, H, eps);                                                  \
+    else if (vec && maxc == 2)                                                                                          \
+      hipLaunchKernelGGL((rmsnorm_vec_kernel<TT, WW, RR, 2>), dim3(T), dim3(vthreads), 0, s, (const TT*)x, (RR*)residual, \
+                         residual_mode, (const WW*)w, (TT*)y, H, eps);                                                  \
+    else                                                                                                                \
+      hipLaunchKernelGGL((rmsnorm_kernel<TT, WW, RR>), dim3(T), dim3(threads), lds, s, (const TT*)x, (RR*)residual,     \
+                         residual_mode, (const WW*)w, (TT*)y, H, eps);                                                  \
+  } while (0)
   if (dtype == NHV_F32 && w_dtype == NHV_F32 && residual_dtype == NHV_F32) LAUNCH(float, float, float);
   else if (dtype == NHV_BF16 && w_dtype == NHV_BF16 && residual_dtype == NHV_F32) LAUNCH(bf16_t, bf16_t, float);
   else if (dtype == NHV_BF16 && w_dtype == NHV_F32 && residual_dtype == NHV_F32) LAUNCH(bf16_t, float, float);

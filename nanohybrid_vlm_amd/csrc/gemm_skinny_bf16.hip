@@ -4,8 +4,8 @@
 //
 // A block owns 16 rows of w (16 outputs n) and all M rows of x. Its waves (2 to 16,
 // more of them where the grid alone would not fill the chip) split K
-// between them in interleaved steps of 32, so that together they read each row of w
-// front to back; a wave's lanes load 16 bytes each straight into the MFMA operand
+// between them in interleaved runs of a few hundred bytes per row, so that together they read each row of w
+// front to back and every cache line is asked for by one wave only; a wave's lanes load 16 bytes each straight into the MFMA operand
 // layout (v_mfma_f32_16x16x32_bf16: w tile as the 16 x 32 operand, x rows as the
 // 32 x 16 one), with several loads in flight before the first is used. The waves'
 // partial sums meet in LDS and are added in the order of the waves, so the result
@@ -24,17 +24,21 @@ __device__ __forceinline__ bf16x8 sk_zero8() {
 }
 
 // MT: tiles of 16 rows of x; WAVES: waves that split K; UNROLL: loads in flight per wave and operand.
-template <int MT, int WAVES, int UNROLL, typename TOut>
+// GLU: w holds two matrices of N rows each, gate above up; the block works on 16 rows of both with the same
+// rows of x and writes silu(gate) * up, so the packed projection's [M, 2N] result never exists in memory.
+template <int MT, int WAVES, int UNROLL, bool GLU, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                  const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                                  int M, int N, int K) {
-  __shared__ float red[WAVES][MT][4][64];
+  constexpr int NA = GLU ? 2 : 1;
+  __shared__ float red[WAVES][NA][MT][4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int n0 = blockIdx.x * 16;
   const int n_a = n0 + col;                          // the row of w that this lane loads
   const bool n_ok = n_a < N;
   const bf16_t* wrow = w + (size_t)(n_ok ? n_a : 0) * K;
+  const bf16_t* wrow2 = wrow + (size_t)N * K;          // GLU: the matching row of the second matrix
   const bf16_t* xrow[MT];
   bool m_ok[MT];
 #pragma unroll
@@ -43,86 +47,127 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(const bf16_t* _
     m_ok[mt] = m < M;
     xrow[mt] = x + (size_t)(m_ok[mt] ? m : 0) * K;
   }
-  floatx4 acc[MT];
+  floatx4 acc[NA][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int na = 0; na < NA; ++na)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[na][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // a wave takes UNROLL consecutive steps of 32 at a time (UNROLL * 64 bytes of every row, whole cache lines),
+  // the waves of the block take such runs in turn
   const int ksteps = (K + 31) / 32;
-  for (int base = wave; base < ksteps; base += WAVES * UNROLL) {
-    bf16x8 a[UNROLL], b[UNROLL][MT];
+  for (int run = wave; run * UNROLL < ksteps; run += WAVES) {
+    bf16x8 a[UNROLL], a2[UNROLL], b[UNROLL][MT];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int k = (base + u * WAVES) * 32 + grp * 8;
+      const int k = (run * UNROLL + u) * 32 + grp * 8;
       const bool k_ok = k < K;                       // K is a multiple of 8: a piece is inside or outside as a whole
       a[u] = (n_ok && k_ok) ? sk_load8(wrow + k) : sk_zero8();
+      if (GLU) a2[u] = (n_ok && k_ok) ? sk_load8(wrow2 + k) : sk_zero8();
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) b[u][mt] = (m_ok[mt] && k_ok) ? sk_load8(xrow[mt] + k) : sk_zero8();
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][mt], acc[mt], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt) {
+        acc[0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][mt], acc[0][mt], 0, 0, 0);
+        if (GLU) acc[NA - 1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[u], b[u][mt], acc[NA - 1][mt], 0, 0, 0);
+      }
   }
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int na = 0; na < NA; ++na)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) red[wave][mt][j][lane] = acc[mt][j];
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) red[wave][na][mt][j][lane] = acc[na][mt][j];
   __syncthreads();
   // the waves share the tiles of the result between them; each sums the partial results in the order of the waves
   for (int mt = wave; mt < MT; mt += WAVES) {
     const int m = mt * 16 + col;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      float v = 0.f;
+      float v = 0.f, v2 = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < WAVES; ++wv) v += red[wv][mt][j][lane];
+      for (int wv = 0; wv < WAVES; ++wv) {
+        v += red[wv][0][mt][j][lane];
+        if (GLU) v2 += red[wv][NA - 1][mt][j][lane];
+      }
       const int n = n0 + grp * 4 + j;               // the tile's row 4 grp + j is output n, its column is row m of x
       if (m < M && n < N) {
         if (bias) v += (float)bias[n];
+        if (GLU) v = v / (1.0f + expf(-v)) * v2;
         y[(size_t)m * N + n] = (TOut)v;
       }
     }
   }
 }
 
-template <int MT, int WAVES, int UNROLL>
+template <int MT, int WAVES, int UNROLL, bool GLU>
 static void sk_launch(unsigned blocks, hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M, int N,
                       int K, int out_dtype) {
   if (out_dtype == NHV_BF16)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, UNROLL, bf16_t>), dim3(blocks), dim3(64 * WAVES), 0, s,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, UNROLL, GLU, bf16_t>), dim3(blocks), dim3(64 * WAVES), 0, s,
                        (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, M, N, K);
   else
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, UNROLL, float>), dim3(blocks), dim3(64 * WAVES), 0, s,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, UNROLL, GLU, float>), dim3(blocks), dim3(64 * WAVES), 0, s,
                        (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (float*)y, M, N, K);
 }
 
-template <int MT, int UNROLL>
+template <int MT, int UNROLL, bool GLU>
 static void sk_by_waves(int waves, unsigned blocks, hipStream_t s, const void* x, const void* w, const void* bias, void* y,
                         int M, int N, int K, int out_dtype) {
-  if (waves >= 16 && MT <= 2) sk_launch<MT, (MT <= 2 ? 16 : 8), UNROLL>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else if (waves >= 8) sk_launch<MT, 8, UNROLL>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else if (waves >= 4) sk_launch<MT, 4, UNROLL>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else sk_launch<MT, 2, UNROLL>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  constexpr int TILES = (GLU ? 2 : 1) * MT;
+  constexpr int MAXW = TILES <= 2 ? 16 : TILES <= 4 ? 8 : 4;      // keeps the block's LDS at 32 KB
+  if (waves >= 16 && MAXW >= 16) sk_launch<MT, (MAXW >= 16 ? 16 : MAXW), UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  else if (waves >= 8 && MAXW >= 8) sk_launch<MT, (MAXW >= 8 ? 8 : MAXW), UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  else if (waves >= 4) sk_launch<MT, 4, UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  else sk_launch<MT, 2, UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
+}
+
+static int sk_check(const char* what, const void* x, const void* w, int M, int N, int K, int out_dtype) {
+  NHV_REQUIRE(M > 0 && N > 0 && K > 0, "%s: bad sizes M=%d N=%d K=%d", what, M, N, K);
+  NHV_REQUIRE(M <= 64, "%s: %d rows are beyond this kernel's limit of 64", what, M);
+  NHV_REQUIRE(K % 8 == 0, "%s: inner size %d must be a multiple of 8", what, K);
+  NHV_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "%s: operands must be 16-byte aligned", what);
+  NHV_REQUIRE(out_dtype == NHV_BF16 || out_dtype == NHV_F32, "%s: unsupported output type %d", what, out_dtype);
+  return 0;
+}
+
+// enough waves in flight to cover the memory's latency: about 16 per compute unit over the whole grid,
+// but no wave with less than one round of loads
+static int sk_waves(unsigned blocks, int K) {
+  const int ksteps = (K + 31) / 32;
+  int waves = 2;
+  while (waves < 16 && (long long)blocks * waves < 4096 && ksteps >= waves * 2 * 4) waves *= 2;
+  return waves;
 }
 
 extern "C" int nhv_gemm_skinny_bf16(const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
                                     int out_dtype, void* stream) {
-  NHV_REQUIRE(M > 0 && N > 0 && K > 0, "skinny gemm: bad sizes M=%d N=%d K=%d", M, N, K);
-  NHV_REQUIRE(M <= 64, "skinny gemm: %d rows are beyond this kernel's limit of 64", M);
-  NHV_REQUIRE(K % 8 == 0, "skinny gemm: inner size %d must be a multiple of 8", K);
-  NHV_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "skinny gemm: operands must be 16-byte aligned");
-  NHV_REQUIRE(out_dtype == NHV_BF16 || out_dtype == NHV_F32, "skinny gemm: unsupported output type %d", out_dtype);
+  if (sk_check("skinny gemm", x, w, M, N, K, out_dtype)) return 1;
   const unsigned blocks = (unsigned)((N + 15) / 16);
   hipStream_t s = (hipStream_t)stream;
   const int mt = (M + 15) / 16;
-  // enough waves in flight to cover the memory's latency: about 16 per compute unit over the whole grid,
-  // but no wave with less than one round of loads
-  const int ksteps = (K + 31) / 32;
-  int waves = 2;
-  while (waves < 16 && (long long)blocks * waves < 4096 && ksteps >= waves * 2 * 4) waves *= 2;
-  if (mt == 1) sk_by_waves<1, 8>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else if (mt == 2) sk_by_waves<2, 8>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else sk_by_waves<4, 4>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  const int waves = sk_waves(blocks, K);
+  if (mt == 1) sk_by_waves<1, 8, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  else if (mt == 2) sk_by_waves<2, 8, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  else sk_by_waves<4, 4, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
   NHV_LAUNCH_CHECK("gemm_skinny_bf16");
+  return 0;
+}
+
+// y[M, N] = silu(x . w[0:N]^T) * (x . w[N:2N]^T): the gated feed-forward's first half in one kernel.
+extern "C" int nhv_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_dtype,
+                                        void* stream) {
+  if (sk_check("skinny gated gemm", x, w, M, N, K, out_dtype)) return 1;
+  const unsigned blocks = (unsigned)((N + 15) / 16);
+  hipStream_t s = (hipStream_t)stream;
+  const int mt = (M + 15) / 16;
+  const int waves = sk_waves(blocks, K);
+  if (mt == 1) sk_by_waves<1, 8, true>(waves, blocks, s, x, w, nullptr, y, M, N, K, out_dtype);
+  else if (mt == 2) sk_by_waves<2, 4, true>(waves, blocks, s, x, w, nullptr, y, M, N, K, out_dtype);
+  else sk_by_waves<4, 4, true>(waves, blocks, s, x, w, nullptr, y, M, N, K, out_dtype);
+  NHV_LAUNCH_CHECK("gemm_skinny_glu_bf16");
   return 0;
 }

@@ -184,6 +184,16 @@ class NativeBackend:
         self._call("nhv_gemm_generic", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K, dtype_code(x),
                    dtype_code(out), _stream())
 
+    def gated_linear(self, x, w, out) -> bool:
+        """silu(x Wg^T) * (x Wu^T) in one kernel, if this batch is one for the few-rows kernel; else False."""
+        M, K = x.shape
+        if (x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+                and (M <= 16 or (M <= 64 and self.own_kernels_only))):
+            self._call("nhv_gemm_skinny_glu_bf16", _ptr(x), _ptr(w), _ptr(out), M, out.shape[1], K, dtype_code(out),
+                       _stream())
+            return True
+        return False
+
     def sample(self, logits, temperatures, keys, tokens):
         n, V = logits.shape
         self._call("nhv_sample", _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(tokens), n, V, _stream())
@@ -341,6 +351,22 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, o
     out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
     backend().linear(x, w, bias, out)
     return out
+
+
+def gated_linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """silu(x . w[:I]^T) * (x . w[I:]^T) for a packed gate | up matrix w[2 I, K]: fused into one kernel for
+    few rows, else the matrix product followed by ``silu_mul``."""
+    _need(x.dim() == 2 and w.dim() == 2 and w.shape[0] % 2 == 0, "gated_linear: x must be [rows, in] and w [2 * out, in]")
+    _need(x.shape[1] == w.shape[1], f"gated_linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
+    _dense(x, "gated_linear: x")
+    _dense(w, "gated_linear: w", dtype=x.dtype)
+    dtype_code(x)
+    fused = getattr(backend(), "gated_linear", None)
+    if fused is not None:
+        out = torch.empty((x.shape[0], w.shape[0] // 2), dtype=x.dtype, device=x.device)
+        if fused(x, w, out):
+            return out
+    return silu_mul(linear(x, w))
 
 
 def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

@@ -26,5 +26,4 @@ class SwiGLU(Part):
         }
 
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
-        gu = ops.linear(x, self.gate_up_weight)
-        return ops.linear(ops.silu_mul(gu), self.down_weight)
+        return ops.linear(ops.gated_linear(x, self.gate_up_weight), self.down_weight)

@@ -44,7 +44,8 @@ def test_embed_and_gather_are_exact(ops, dtype, T, H, V):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,H,eps", [(3, 80, 1e-5), (17, 1000, 1e-6), (5, 4096, 1e-6), (2, 12288, 1e-3)])
+@pytest.mark.parametrize("T,H,eps", [(3, 80, 1e-5), (17, 1000, 1e-6), (5, 4096, 1e-6), (2, 12288, 1e-3), (4, 1001, 1e-5),
+                                     (1, 8192, 1e-6), (300, 5120, 1e-6), (2, 16368, 1e-6)])
 def test_rmsnorm(ops, dtype, T, H, eps):
     x = rnd(T, H, dtype=dtype, seed=1, scale=3.0)
     w = (1 + 0.1 * torch.randn(H)).to(dtype).cuda()
@@ -124,6 +125,18 @@ def test_skinny_linear_bfloat16(ops, M, N, K):
     if M > 1:
         torch.testing.assert_close(ops.linear(x[:1].contiguous(), w, out_dtype=torch.float32),
                                    ops.linear(x, w, out_dtype=torch.float32)[:1], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 112, 80), (5, 1001, 96), (16, 12288, 4096), (17, 160, 96), (64, 300, 1024)])
+def test_gated_linear(ops, M, I, K):
+    """silu(x Wg^T) * (x Wu^T): the fused kernel for few rows, the two-kernel way for many; float32 as well."""
+    for dtype in DTYPES:
+        x = rnd(M, K, dtype=dtype, seed=24)
+        w = rnd(2 * I, K, dtype=dtype, seed=25, scale=K ** -0.5)
+        g, u = x.double() @ w[:I].double().T, x.double() @ w[I:].double().T
+        ref = g * torch.sigmoid(g) * u
+        t = dict(rtol=1e-5, atol=2e-5) if dtype == torch.float32 else tol(dtype)
+        torch.testing.assert_close(ops.gated_linear(x, w).double(), ref, **t)
 
 
 def test_linear_rows_do_not_depend_on_the_batch_in_float32(ops):

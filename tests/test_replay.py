@@ -115,6 +115,29 @@ def test_replay_on_gpu(model_folders, name, dtype, graphs, tmp_path):
                 assert d <= 2e-6, f"float32 {mode} against whole: request {rid}: {d:.3e}"
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(model_folders, dtype, graphs):
+    """One token a step from the very first token on, 500 steps, two requests side by side that start at
+    different times: every page edge, every split edge of the decode kernel and the first positions."""
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    folder = model_folders["B"]
+    cfg, w = plain.read_model_folder(folder)
+    a = rc.random_tokens(cfg["vocab_size"], 500, 1)
+    b = rc.random_tokens(cfg["vocab_size"], 300, 2)
+    steps = []
+    for i in range(500):
+        entries = [{"id": "a", "tokens": [a[i]], "want": [0]}]
+        if 100 <= i < 400:
+            entries.append({"id": "b", "tokens": [b[i - 100]], "want": [0]})
+        steps.append({"step": i, "entries": entries, "end": (["a"] if i == 499 else []) + (["b"] if i == 399 else [])})
+    runner = ModelRunner(folder, dtype=dtype, page_size=8, num_pages=101, num_state_slots=2, use_graphs=graphs,
+                         max_model_len=512)
+    got = rc.run_in_process(runner, steps)
+    _check(got, {"a": plain.logits(cfg, w, a), "b": plain.logits(cfg, w, b)}, TOLERANCE[dtype], f"{dtype} long decoding")
+
+
 def _trace_run(folder, dtype, steps, out_dir, max_tokens, extra=()):
     cmd = [sys.executable, os.path.join(REPO, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
            "--out", out_dir, "--max-tokens", str(max_tokens), *extra]
