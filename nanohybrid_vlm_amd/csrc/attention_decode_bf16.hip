@@ -26,7 +26,9 @@ constexpr int DSTEPS = (D + 31) / 32;                       // MFMA steps over t
 constexpr int CHUNKS = D / 8;                               // 16-byte pieces of a row
 constexpr int LPK = CHUNKS <= 2 ? 2 : CHUNKS <= 4 ? 4 : CHUNKS <= 8 ? 8 : CHUNKS <= 16 ? 16 : CHUNKS <= 32 ? 32 : 64;
 constexpr int KPP = 64 / LPK;                               // keys per pass of the value half
-constexpr int PASSES = 16 / KPP > 0 ? 16 / KPP : 1;
+constexpr int RK = 64;                                      // keys per round
+constexpr int KT = RK / 16;                                 // MFMA tiles of 16 keys per round
+constexpr int PASSES = RK / KPP;                            // passes of the value half per round
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -39,13 +41,19 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// key position -> slot in the cache; pages whose size is a power of two need no division
+__device__ __forceinline__ int slot_of(const int* bt, int key, int page_size, int page_shift) {
+  if (page_shift >= 0) return (bt[key >> page_shift] << page_shift) + (key & (page_size - 1));
+  return bt[key / page_size] * page_size + key % page_size;
+}
+
 template <int GC>
 __global__ __launch_bounds__(64) void decode_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     float* __restrict__ part_o, float* __restrict__ part_ml, const int* __restrict__ token_req,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv,
-    int page_size, float scale, int window, int split_len, int n_splits) {
-  __shared__ float p_s[16][17];          // [key][head]
+    int page_size, int page_shift, float scale, int window, int split_len, int n_splits) {
+  __shared__ __attribute__((aligned(16))) float p_s[RK][20];          // [key][head], rows of 16-byte pieces
   __shared__ float alpha_s[16];
   const int lane = threadIdx.x;
   const int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
@@ -75,67 +83,67 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
   const int ksub = lane / LPK, chunk = lane % LPK;
   const bool chunk_live = chunk * 8 < D;
 
-  // keys of one round, as the first product's operand: lane loads 8 entries of key kb + col
-  auto load_keys = [&](int kb, bf16x8* ka) {
-    const int key = kb + col;
-    const bool ok = key >= first && key <= last;
-    int slot = 0;
-    if (ok) slot = bt[key / page_size] * page_size + key % page_size;
-    const bf16_t* krow = k_cache + ((size_t)slot * Hkv + kvh) * D;
+  for (int kb = (first / RK) * RK; kb <= last; kb += RK) {
+    // ---- all keys and values of the round are asked for before anything is computed: 64 keys, 32 KB a wave
+    // (pages that are a power of two of at least 64 tokens hold a whole round: one look at the block table)
+    const bool one_page = page_shift >= 6;
+    const int round_base = one_page ? (bt[kb >> page_shift] << page_shift) : 0;
+    bf16x8 ka[KT][DSTEPS];
 #pragma unroll
-    for (int s = 0; s < DSTEPS; ++s) {
-      const int d = s * 32 + grp * 8;
-      ka[s] = (ok && d < D) ? load8(krow + d) : zero8();
+    for (int kt = 0; kt < KT; ++kt) {
+      const int key = kb + kt * 16 + col;
+      const bool ok = key >= first && key <= last;
+      int slot = 0;
+      if (ok) slot = one_page ? round_base + (key & (page_size - 1)) : slot_of(bt, key, page_size, page_shift);
+      const bf16_t* krow = k_cache + ((size_t)slot * Hkv + kvh) * D;
+#pragma unroll
+      for (int s = 0; s < DSTEPS; ++s) {
+        const int d = s * 32 + grp * 8;
+        ka[kt][s] = (ok && d < D) ? load8(krow + d) : zero8();
+      }
     }
-  };
-
-  const int kb0 = (first / 16) * 16;
-  bf16x8 ka[DSTEPS];
-  load_keys(kb0, ka);
-  for (int kb = kb0; kb <= last; kb += 16) {
-    // ---- this round's values and the next round's keys are asked for before anything is computed
     bf16x8 vv[PASSES];
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-      const int kl = ps * KPP + ksub;
-      const int key = kb + kl;
-      const bool ok = chunk_live && kl < 16 && key >= first && key <= last;
+      const int key = kb + ps * KPP + ksub;
+      const bool ok = chunk_live && key >= first && key <= last;
       int slot = 0;
-      if (ok) slot = bt[key / page_size] * page_size + key % page_size;
+      if (ok) slot = one_page ? round_base + (key & (page_size - 1)) : slot_of(bt, key, page_size, page_shift);
       vv[ps] = ok ? load8(v_cache + ((size_t)slot * Hkv + kvh) * D + chunk * 8) : zero8();
     }
-    bf16x8 kn[DSTEPS];
-    if (kb + 16 <= last) {
-      load_keys(kb + 16, kn);
-    } else {
+    // ---- scores
+    floatx4 s4[KT];
 #pragma unroll
-      for (int s = 0; s < DSTEPS; ++s) kn[s] = zero8();
+    for (int kt = 0; kt < KT; ++kt) {
+      s4[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < DSTEPS; ++s) s4[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kt][s], qb[s], s4[kt], 0, 0, 0);
     }
-    // ---- scores of 16 keys
-    floatx4 s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < DSTEPS; ++s) s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[s], qb[s], s4, 0, 0, 0);
-    // ---- running softmax for head `col` over keys kb + 4 grp + j
-    float sc[4];
+    // ---- running softmax for head `col` over keys kb + 16 kt + 4 grp + j
     float m_tile = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int key = kb + grp * 4 + j;
-      sc[j] = (key >= first && key <= last) ? s4[j] * scale : -INFINITY;
-      m_tile = fmaxf(m_tile, sc[j]);
-    }
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int key = kb + kt * 16 + grp * 4 + j;
+        const float v = (key >= first && key <= last) ? s4[kt][j] * scale : -INFINITY;
+        s4[kt][j] = v;
+        m_tile = fmaxf(m_tile, v);
+      }
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
     const float m_new = fmaxf(m_run, m_tile);          // finite: every round holds a visible key
-    const float alpha = expf(m_run - m_new);
+    const float alpha = __expf(m_run - m_new);
     float psum = 0.f;
     __syncthreads();                                   // the last round's p_s and alpha_s have been read
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float p = expf(sc[j] - m_new);             // exp(-inf) = 0 for keys out of range
-      p_s[grp * 4 + j][col] = p;
-      psum += p;
-    }
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float p = __expf(s4[kt][j] - m_new);     // exp(-inf) = 0 for keys out of range
+        p_s[kt * 16 + grp * 4 + j][col] = p;
+        psum += p;
+      }
     l_part = l_part * alpha + psum;
     m_run = m_new;
     if (grp == 0) alpha_s[col] = alpha;
@@ -150,20 +158,25 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
       const int kl = ps * KPP + ksub;
-      if (kl < 16) {
-        float vf[8];
+      float vf[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) vf[e] = (float)vv[ps][e];
+      for (int e = 0; e < 8; ++e) vf[e] = (float)vv[ps][e];
+      float pg[GC];
+      if (GC >= 4) {
 #pragma unroll
-        for (int g = 0; g < GC; ++g) {
-          const float p = p_s[kl][g];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(p, vf[e], acc[g][e]);
+        for (int g4 = 0; g4 < GC / 4; ++g4) {
+          const float4 p4 = *reinterpret_cast<const float4*>(&p_s[kl][g4 * 4]);
+          pg[g4 * 4] = p4.x; pg[g4 * 4 + 1] = p4.y; pg[g4 * 4 + 2] = p4.z; pg[g4 * 4 + 3] = p4.w;
         }
-      }
-    }
+      } else {
 #pragma unroll
-    for (int s = 0; s < DSTEPS; ++s) ka[s] = kn[s];
+        for (int g = 0; g < GC; ++g) pg[g] = p_s[kl][g];
+      }
+#pragma unroll
+      for (int g = 0; g < GC; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pg[g], vf[e], acc[g][e]);
+    }
   }
   // ---- this split's result: sum over the lanes that hold other keys of the same chunk
 #pragma unroll
@@ -264,10 +277,13 @@ extern "C" int nhv_decode_attention_bf16(const void* q, const void* k_cache, con
                                          const void* block_tables, int max_blocks, int T, int Hq, int Hkv, int page_size,
                                          float scale, int window, int split_len, int n_splits, void* stream) {
   NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && page_size > 0 && max_blocks > 0, "decode attention: bad sizes");
+  int page_shift = -1;
+  for (int b = 0; b < 31; ++b)
+    if (page_size == (1 << b)) page_shift = b;
   NHV_REQUIRE(Hq % Hkv == 0, "decode attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   const int G = Hq / Hkv;
   NHV_REQUIRE(G <= 16, "decode attention: %d query heads per key head are beyond this kernel's limit of 16", G);
-  NHV_REQUIRE(split_len > 0 && split_len % 16 == 0, "decode attention: split length %d must be a multiple of 16", split_len);
+  NHV_REQUIRE(split_len > 0 && split_len % RK == 0, "decode attention: split length %d must be a multiple of %d", split_len, RK);
   NHV_REQUIRE(n_splits > 0 && n_splits <= 65535 && Hkv <= 65535 && T <= 65535, "decode attention: grid too large");
   NHV_REQUIRE(window >= 0, "decode attention: negative window");
   hipStream_t s = (hipStream_t)stream;
@@ -275,8 +291,8 @@ extern "C" int nhv_decode_attention_bf16(const void* q, const void* k_cache, con
 #define LAUNCH(GC)                                                                                                    \
   hipLaunchKernelGGL(decode_attention_kernel<GC>, grid, dim3(64), 0, s, (const bf16_t*)q, (const bf16_t*)k_cache,     \
                      (const bf16_t*)v_cache, (float*)part_o, (float*)part_ml, (const int*)token_req,                  \
-                     (const int*)positions, (const int*)block_tables, max_blocks, Hq, Hkv, page_size, scale, window,  \
-                     split_len, n_splits)
+                     (const int*)positions, (const int*)block_tables, max_blocks, Hq, Hkv, page_size, page_shift, scale,   \
+                     window, split_len, n_splits)
   if (G <= 1) LAUNCH(1);
   else if (G <= 2) LAUNCH(2);
   else if (G <= 4) LAUNCH(4);

@@ -132,7 +132,7 @@ class NativeBackend:
     def paged_attention(self, q, k_cache, v_cache, out, batch: AttentionBatch, block_tables, scale, window):
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
-        if (q.dtype == torch.bfloat16 and batch.max_q_len == 1 and D % 16 == 0 and D <= 512 and Hq // Hkv <= 16
+        if (q.dtype == torch.bfloat16 and batch.max_q_len == 1 and D % 16 == 0 and D <= 256 and Hq // Hkv <= 16
                 and T <= 65535):
             return self._decode_attention(q, k_cache, v_cache, out, batch, block_tables, scale, window)
         if q.dtype == torch.bfloat16 and D % 16 == 0 and D <= 256 and batch.num_requests <= 65535 and Hkv <= 65535:
@@ -149,9 +149,12 @@ class NativeBackend:
         """Single tokens in bfloat16: keys split over waves, then merged."""
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
-        span = batch.max_context_len if not window else min(batch.max_context_len, window + 16)
-        # enough waves to fill the chip (about 1024 of them), each with enough keys to be worth its start
-        want = max(1, T * Hkv * span // 1024)
+        # inside a graph the lengths are only bounded (by max_model_len): plan for half the bound
+        span = batch.max_context_len // 2 if self.own_kernels_only else batch.max_context_len
+        if window:
+            span = min(span, window + 64)
+        # enough waves to fill the chip's 1024 SIMDs twice over, each with at least one round of 64 keys
+        want = max(1, T * Hkv * span // 2048)
         split_len = 64
         while split_len < want and split_len < 1024:
             split_len *= 2

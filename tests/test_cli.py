@@ -1,0 +1,42 @@
+"""The command line, started as a user would."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+import plain_qwen3 as plain
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _run(*args, timeout=600):
+    proc = subprocess.run([sys.executable, "-m", "nanohybrid_vlm_amd", *args], cwd=REPO, capture_output=True, text=True,
+                          timeout=timeout)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    return proc.stdout
+
+
+def test_random_model_command(tmp_path):
+    out = str(tmp_path / "m")
+    _run("random-model", "--out", out, "--shape", "tinyB", "--seed", "3")
+    cfg, w = plain.read_model_folder(out)
+    assert cfg["hidden_size"] == 96 and "lm_head.weight" in w
+    assert plain.logits(cfg, w, [1, 2, 3]).shape == (3, 389)
+
+
+@pytest.mark.gpu
+def test_generate_and_bench_commands(model_folders, tmp_path):
+    folder = model_folders["A"]
+    cfg, w = plain.read_model_folder(folder)
+    out = json.loads(_run("generate", "--model", folder, "--dtype", "float32", "--prompt-ids", "5 17 3", "--prompt-ids",
+                          "9,8,7,6", "--output-tokens", "5", "--temperature", "0", "--ignore-eos", "--block-size", "8",
+                          "--num-blocks", "16", "--max-model-len", "64", "--quiet"))
+    assert [o["token_ids"] for o in out] == [plain.greedy_generate(cfg, w, p, 5) for p in ([5, 17, 3], [9, 8, 7, 6])]
+    result = str(tmp_path / "bench.json")
+    _run("bench", "--model", folder, "--cases", "16:2", "40:3", "--output-tokens", "6", "--repeats", "1",
+         "--warmup-output-tokens", "2", "--token-budget", "32", "--block-size", "8", "--num-blocks", "64",
+         "--max-model-len", "128", "--label", "tiny", "--mode", "graph", "--output", result)
+    data = json.loads(open(result).read())
+    assert len(data["results"]) == 2 and all(r["decode_tok_s"] > 0 and r["ttft_ms_mean"] > 0 for r in data["results"])
