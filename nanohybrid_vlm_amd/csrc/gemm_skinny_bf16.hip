@@ -125,6 +125,129 @@ static void sk_by_waves(int waves, unsigned blocks, hipStream_t s, const void* x
   else sk_launch<MT, 2, UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
 }
 
+// For 17 to 64 rows of x the rows of x are the larger share of what a wave loads, so here a wave keeps NT
+// tiles of 16 rows of w (and with GLU their partners in the second matrix) against the same rows of x:
+// every load of x serves NT (2 NT) products. The partial sums of the waves meet in LDS one tile at a time.
+template <int MT, int NT, int WAVES, int UNROLL, bool GLU, typename TOut>
+__global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                              const bf16_t* __restrict__ bias, TOut* __restrict__ y,
+                                                              int M, int N, int K) {
+  constexpr int NA = GLU ? 2 : 1;
+  constexpr int TILES = NA * NT;
+  static_assert(MT <= WAVES, "each of the first MT waves finishes one tile of rows of x");
+  __shared__ float red[WAVES][MT][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int n0 = blockIdx.x * 16 * NT;
+  const bf16_t* wrow[TILES];
+  bool n_ok[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = n0 + nt * 16 + col;
+    n_ok[nt] = n < N;
+#pragma unroll
+    for (int na = 0; na < NA; ++na) wrow[na * NT + nt] = w + ((size_t)na * N + (n_ok[nt] ? n : 0)) * K;
+  }
+  const bf16_t* xrow[MT];
+  bool m_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + col;
+    m_ok[mt] = m < M;
+    xrow[mt] = x + (size_t)(m_ok[mt] ? m : 0) * K;
+  }
+  floatx4 acc[TILES][MT];
+#pragma unroll
+  for (int t = 0; t < TILES; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int ksteps = (K + 31) / 32;
+  for (int run = wave; run * UNROLL < ksteps; run += WAVES) {
+    bf16x8 a[UNROLL][TILES], b[UNROLL][MT];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int k = (run * UNROLL + u) * 32 + grp * 8;
+      const bool k_ok = k < K;
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) a[u][t] = (n_ok[t % NT] && k_ok) ? sk_load8(wrow[t] + k) : sk_zero8();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) b[u][mt] = (m_ok[mt] && k_ok) ? sk_load8(xrow[mt] + k) : sk_zero8();
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][t], b[u][mt], acc[t][mt], 0, 0, 0);
+  }
+  // wave `mt` adds the waves' partial sums of tile (t, mt) in the order of the waves and writes that tile
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    float v[NA][4];
+#pragma unroll
+    for (int na = 0; na < NA; ++na) {
+      __syncthreads();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) red[wave][mt][j][lane] = acc[na * NT + nt][mt][j];
+      __syncthreads();
+      if (wave < MT) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float sum = 0.f;
+#pragma unroll
+          for (int wv = 0; wv < WAVES; ++wv) sum += red[wv][wave][j][lane];
+          v[na][j] = sum;
+        }
+      }
+    }
+    if (wave < MT) {
+      const int m = wave * 16 + col;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + nt * 16 + grp * 4 + j;
+        if (m < M && n < N) {
+          float r = v[0][j];
+          if (bias) r += (float)bias[n];
+          if (GLU) r = r / (1.0f + expf(-r)) * v[NA - 1][j];
+          y[(size_t)m * N + n] = (TOut)r;
+        }
+      }
+    }
+  }
+}
+
+template <int MT, int NT, bool GLU>
+static void mid_launch(hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
+                       int out_dtype) {
+  constexpr int WAVES = 8, UNROLL = 2;
+  const unsigned blocks = (unsigned)((N + 16 * NT - 1) / (16 * NT));
+  if (out_dtype == NHV_BF16)
+    hipLaunchKernelGGL((gemm_mid_kernel<MT, NT, WAVES, UNROLL, GLU, bf16_t>), dim3(blocks), dim3(64 * WAVES), 0, s,
+                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_mid_kernel<MT, NT, WAVES, UNROLL, GLU, float>), dim3(blocks), dim3(64 * WAVES), 0, s,
+                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (float*)y, M, N, K);
+}
+
+// more than 16 rows: how many tiles of w a wave keeps, by how many blocks that leaves for the chip
+template <bool GLU>
+static void mid_dispatch(hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
+                         int out_dtype) {
+  const int mt = (M + 15) / 16;
+  const bool wide = !GLU && N >= 16384;
+  if (mt == 2) {
+    if (wide) mid_launch<2, 4, GLU>(s, x, w, bias, y, M, N, K, out_dtype);
+    else mid_launch<2, 2, GLU>(s, x, w, bias, y, M, N, K, out_dtype);
+  } else {
+    if (wide) mid_launch<4, 4, GLU>(s, x, w, bias, y, M, N, K, out_dtype);
+    else mid_launch<4, 2, GLU>(s, x, w, bias, y, M, N, K, out_dtype);
+  }
+}
+
 static int sk_check(const char* what, const void* x, const void* w, int M, int N, int K, int out_dtype) {
   NHV_REQUIRE(M > 0 && N > 0 && K > 0, "%s: bad sizes M=%d N=%d K=%d", what, M, N, K);
   NHV_REQUIRE(M <= 64, "%s: %d rows are beyond this kernel's limit of 64", what, M);
@@ -149,8 +272,15 @@ extern "C" int nhv_gemm_skinny_bf16(const void* x, const void* w, const void* bi
   const unsigned blocks = (unsigned)((N + 15) / 16);
   hipStream_t s = (hipStream_t)stream;
   const int mt = (M + 15) / 16;
+  if (mt >= 2) {
+    mid_dispatch<false>(s, x, w, bias, y, M, N, K, out_dtype);
+    NHV_LAUNCH_CHECK("gemm_mid_bf16");
+    return 0;
+  }
   const int waves = sk_waves(blocks, K);
-  if (mt == 1) sk_by_waves<1, 8, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  // long runs per wave (1 KB of every row in flight) where K is long enough to give every wave two of them
+  if (mt == 1 && (K + 31) / 32 >= waves * 32) sk_by_waves<1, 16, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
+  else if (mt == 1) sk_by_waves<1, 8, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
   else if (mt == 2) sk_by_waves<2, 8, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
   else sk_by_waves<4, 4, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
   NHV_LAUNCH_CHECK("gemm_skinny_bf16");
@@ -164,6 +294,11 @@ extern "C" int nhv_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, i
   const unsigned blocks = (unsigned)((N + 15) / 16);
   hipStream_t s = (hipStream_t)stream;
   const int mt = (M + 15) / 16;
+  if (mt >= 2) {
+    mid_dispatch<true>(s, x, w, nullptr, y, M, N, K, out_dtype);
+    NHV_LAUNCH_CHECK("gemm_mid_glu_bf16");
+    return 0;
+  }
   const int waves = sk_waves(blocks, K);
   if (mt == 1) sk_by_waves<1, 8, true>(waves, blocks, s, x, w, nullptr, y, M, N, K, out_dtype);
   else if (mt == 2) sk_by_waves<2, 4, true>(waves, blocks, s, x, w, nullptr, y, M, N, K, out_dtype);

@@ -46,7 +46,7 @@ class ModelRunner:
     def __init__(self, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 256,
                  num_pages: int | None = None, num_state_slots: int = 512, gpu_memory_utilization: float = 0.9,
                  max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None, use_graphs: bool = False,
-                 max_model_len: int | None = None, max_graph_batch: int = 64):
+                 max_model_len: int | None = None, max_graph_batch: int = 16):
         """``model``/``arch``/``cfg`` may be given ready-made (weights already bound)
         instead of being read from ``model_dir``."""
         if dtype not in _TORCH_DTYPES:
@@ -68,7 +68,9 @@ class ModelRunner:
         self._pinned = None
         self._pinned_free = None
         # decode-only steps replay a HIP graph per batch-size bucket (the reference captures CUDA graphs for
-        # the same batch sizes, nanovllm/engine/model_runner.py:2559-2594)
+        # the same batch sizes, nanovllm/engine/model_runner.py:2559-2594). Up to 16 requests a step is bound
+        # by launches and by the own few-rows kernels; larger batches run eagerly, where the matrix products
+        # of 17 and more rows are the library's (measured faster than the own kernel at those sizes)
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
         self.max_model_len = min(max_model_len or self.max_position, self.max_position)
         self.max_graph_batch = max_graph_batch
