@@ -2,20 +2,25 @@
 // cache in bfloat16 on the matrix cores. Compiled for one head size:
 // -DNHV_HEAD_DIM=<multiple of 16>.
 //
-// A block of 4 waves works on one (request, key/value head) and four row tiles; a row
-// tile is 16 consecutive tokens of one query head, and the row tiles of a request are
-// numbered so that the heads sharing the key/value head come first: with 4 heads per
-// key/value head a block is 16 tokens x 4 heads, and every key and value it stages
-// in LDS is used by 64 rows. Keys are taken in tiles of 64, in rising order:
-//   S^T[key, row] = K[key, :] . Q[row, :]     K tile from LDS, Q in registers (v_mfma_f32_16x16x32_bf16)
-//   running maximum and sum per row in float (two shuffles over the lane groups)
-//   O[row, d]   += P[row, key] . V[key, d]    P from registers, V^T from LDS (v_mfma_f32_16x16x16_bf16)
-// The S^T tile leaves every lane with four consecutive keys of one row, which is the
-// operand layout of the second product, so P never goes through memory. V is
-// written to LDS transposed, so that its operand is one 8-byte read.
-// A query at position p reads keys lo..p (lo = p - window + 1 with a window, else 0).
-// Keys outside the block's range are staged as zeros: unused cache slots may hold
-// anything, and 0 * NaN would poison the sums.
+// A block of 4 waves works on one (request, key/value head) and four row tiles, one per
+// wave; a row tile is 16 consecutive tokens of one query head, and the row tiles of a
+// request are numbered so that the heads sharing the key/value head come first: with 4
+// heads per key/value head a block is 16 tokens x 4 heads, and every key and value it
+// stages in LDS is used by 64 rows. Keys are taken in tiles of 64, in rising order:
+//   S^T[key, row] = K[key, :] . Q[row, :]      K tile from LDS, Q in registers (v_mfma_f32_16x16x32_bf16)
+//   running maximum per row in float (two shuffles over the lane groups), sums kept per lane
+//   O^T[d, row]  += V^T[d, key] . P^T[key, row]  V^T from LDS, P in registers (v_mfma_f32_16x16x32_bf16)
+// An S^T tile leaves every lane with four consecutive keys of one row; two such tiles
+// side by side are the eight summation slots of a lane in the second product (the
+// order of the slots is free as long as P and V agree), so P never goes through
+// memory, and because the second product is taken transposed a lane's output entries
+// belong to the same row as its scores: the rescaling needs no exchange between lanes.
+// V is written to LDS transposed, four keys (8 bytes) at a time; the columns of that
+// tile are XOR-ed with the row's 8-group so that a wave's writes fall into distinct banks.
+// The next tile's keys and values are asked for from memory before the current tile
+// is computed. A query at position p reads keys lo..p (lo = p - window + 1 with a
+// window, else 0). Keys outside the block's range are staged as zeros: unused cache
+// slots may hold anything, and 0 * NaN would poison the sums.
 #include "nhv_common.h"
 #include <math.h>
 
@@ -35,6 +40,10 @@ constexpr int BN = D <= 128 ? 64 : 32;      // keys per tile
 constexpr int KT = BN / 16;                 // 16-key sub-tiles
 constexpr int KPITCH = DSTEPS * 32 + 8;     // elements per row of the K tile (padded against bank conflicts)
 constexpr int VPITCH = BN + 8;              // elements per row of the transposed V tile
+constexpr int QUADS = (BN / 4) * CH;        // (4 keys, 16-byte piece) units of a tile
+constexpr int QPT = (QUADS + 255) / 256;    // of them per thread
+constexpr int SWZ_MASK = BN / 4 - 1;        // column of key k in row d of the V^T tile: k ^ (((d >> 3) & SWZ_MASK) << 2)
+constexpr int TPB = 4;                      // row tiles per block, one per wave
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
@@ -47,13 +56,26 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+constexpr int BT_LDS = 1024;                // block-table entries that are kept in LDS
+
+template <typename P>
+__device__ __forceinline__ int slot_of(P bt, int key, int page_size, int page_shift) {
+  if (page_shift >= 0) return (bt[key >> page_shift] << page_shift) + (key & (page_size - 1));
+  return bt[key / page_size] * page_size + key % page_size;
+}
+
+// BT_IN_LDS: the request's block table (up to the block's last key) is copied into LDS first, so that the
+// look-up that every load of a key depends on costs an LDS read instead of a trip to memory.
+template <bool BT_IN_LDS>
 __global__ __launch_bounds__(256) void prefill_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens_q, const int* __restrict__ context_lens,
-    const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv, int page_size, float scale, int window) {
+    const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv, int page_size, int page_shift,
+    float scale_log2e, int window) {
   constexpr int DL = SUPPORTED ? D : 16;                   // keeps the unsupported sizes compilable; they are never launched
   __shared__ __attribute__((aligned(16))) bf16_t k_s[BN * (SUPPORTED ? KPITCH : 24)];
   __shared__ __attribute__((aligned(16))) bf16_t vt_s[DL * VPITCH];
+  __shared__ int bt_s[BT_IN_LDS ? BT_LDS : 1];
   if (!SUPPORTED) return;
 
   const int req = blockIdx.z, kvh = blockIdx.y;
@@ -63,29 +85,38 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
   const int ctx = context_lens[req];
   const int start_pos = ctx - q_len;                       // position of the request's first token in this step
   const int n_row_tiles = G * ((q_len + 15) / 16);
-  const int first_tile = blockIdx.x * 4;
+  // Causal work grows with the row tile's place in the portion, and all blocks of a long portion are resident
+  // at once, so which blocks share a compute unit decides the kernel's time. Blocks 256 apart in launch order
+  // (256 compute units) tend to land on the same unit: every second such round takes its row tiles from the
+  // other end of the portion, so that a unit's blocks have long and short key ranges in turn.
+  // (A whole row of the grid turns together, so that every row tile is still taken exactly once.)
+  const int row_launch_index = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x;
+  const int bx = ((row_launch_index >> 8) & 1) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  const int first_tile = bx * TPB;
   if (first_tile >= n_row_tiles) return;                   // the grid is made for the longest portion of the batch
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const int my_tile = first_tile + wave;
-  const bool wave_live = my_tile < n_row_tiles;
-  const int head = kvh * G + (wave_live ? my_tile % G : 0);
-  const int tok0 = wave_live ? (my_tile / G) * 16 : 0;     // first token (within the portion) of this wave's rows
 
   // the block's key range: from the smallest lower bound to the largest position of its rows
-  const int last_tile = min(first_tile + 3, n_row_tiles - 1);
+  const int last_tile = min(first_tile + TPB - 1, n_row_tiles - 1);
   const int blk_tok_lo = (first_tile / G) * 16;
   const int blk_tok_hi = min((last_tile / G) * 16 + 15, q_len - 1);
   const int key_hi = start_pos + blk_tok_hi;
   const int key_lo = window > 0 ? max(0, start_pos + blk_tok_lo - window + 1) : 0;
 
-  // this lane's row in the first product: token tok0 + col
+  // this wave's row tile; this lane's row (in both products) is token tok0 + col of the tile's head
+  const int my_tile = first_tile + wave;
+  const bool live = my_tile < n_row_tiles;
+  const int head = kvh * G + (live ? my_tile % G : 0);
+  const int tok0 = live ? (my_tile / G) * 16 : 0;
   const int row_tok = tok0 + col;
-  const bool row_ok = wave_live && row_tok < q_len;
+  const bool row_ok = live && row_tok < q_len;
   const int row_pos = start_pos + min(row_tok, q_len - 1);
   const int row_lo = window > 0 ? max(0, row_pos - window + 1) : 0;
-  const int wave_hi = start_pos + min(tok0 + 15, q_len - 1);   // beyond it this wave has nothing to do
+  const int wave_lo_pos = start_pos + tok0;                    // the tile's first row sees the fewest keys
+  const int wave_hi = start_pos + min(tok0 + 15, q_len - 1);   // beyond it this tile has nothing to do
+  const int wave_max_lo = window > 0 ? max(0, wave_hi - window + 1) : 0;
 
   bf16x8 qb[DSTEPS];
 #pragma unroll
@@ -94,37 +125,84 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
     qb[s] = (row_ok && d < D) ? *reinterpret_cast<const bf16x8*>(q + ((size_t)(q_begin + row_tok) * Hq + head) * D + d)
                               : zero8();
   }
-
-  float m_run = -INFINITY, l_run = 0.f;                    // of row `col`, the same in all four lane groups
-  floatx4 o[DTILES];                                       // o[dt][j]: row 4 grp + j, column dt * 16 + col
+  float m_run = -INFINITY;                                 // of row `col`, the same in all four lane groups (base 2)
+  float l_part = 0.f;                                      // this lane's share of the row's sum
+  floatx4 o[DTILES];                                       // o[dt][j]: entry dt * 16 + 4 grp + j of row `col`
 #pragma unroll
   for (int dt = 0; dt < DTILES; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const int* bt = block_tables + (size_t)req * max_blocks;
-
-  for (int kb = (key_lo / BN) * BN; kb <= key_hi; kb += BN) {
-    __syncthreads();                                       // the last tile has been read by every wave
-    // ---- stage 64 keys and values
-    for (int c = tid; c < BN * CH; c += 256) {
-      const int kl = c / CH, dc = c % CH;
-      const int key = kb + kl;
-      bf16x8 kv8 = zero8(), vv8 = zero8();
-      if (key >= key_lo && key <= key_hi) {
-        const int slot = bt[key / page_size] * page_size + key % page_size;
-        const size_t off = ((size_t)slot * Hkv + kvh) * D + dc * 8;
-        kv8 = *reinterpret_cast<const bf16x8*>(k_cache + off);
-        vv8 = *reinterpret_cast<const bf16x8*>(v_cache + off);
-      }
-      *reinterpret_cast<bf16x8*>(k_s + kl * KPITCH + dc * 8) = kv8;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) vt_s[(dc * 8 + e) * VPITCH + kl] = vv8[e];
-    }
-    if (D % 32 != 0) {                                     // the padded half step of the first product reads zeros
-      for (int c = tid; c < BN * 2; c += 256) *reinterpret_cast<bf16x8*>(k_s + (c / 2) * KPITCH + D + (c % 2) * 8) = zero8();
-    }
+  const int* bt_g = block_tables + (size_t)req * max_blocks;
+  if (BT_IN_LDS) {
+    const int n_entries = min(BT_LDS, key_hi / page_size + 1);
+    for (int i = tid; i < n_entries; i += 256) bt_s[i] = bt_g[i];
     __syncthreads();
-    if (!wave_live || kb > wave_hi) continue;              // whole wave; it still meets the others at the barriers
+  }
+  // where the key look-ups go: LDS copy or memory
+  auto slot = [&](int key) {
+    return BT_IN_LDS ? slot_of((const int*)bt_s, key, page_size, page_shift) : slot_of(bt_g, key, page_size, page_shift);
+  };
 
+  // staging: a thread owns the same 16-byte piece of four consecutive keys
+  bf16x8 kreg[QPT][4], vreg[QPT][4];
+  auto fetch = [&](int kb) {                               // memory -> registers
+    const bool whole = kb >= key_lo && kb + BN - 1 <= key_hi;    // every key of the tile is in range (all but the ends)
+#pragma unroll
+    for (int i = 0; i < QPT; ++i) {
+      const int u = tid + i * 256;
+      const int kq = u / CH, dc = u % CH;
+      if (whole && (QUADS % 256 == 0 || u < QUADS)) {
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) {
+          const size_t off = ((size_t)slot(kb + kq * 4 + k4) * Hkv + kvh) * D + dc * 8;
+          kreg[i][k4] = *reinterpret_cast<const bf16x8*>(k_cache + off);
+          vreg[i][k4] = *reinterpret_cast<const bf16x8*>(v_cache + off);
+        }
+        continue;
+      }
+#pragma unroll
+      for (int k4 = 0; k4 < 4; ++k4) {
+        const int key = kb + kq * 4 + k4;
+        kreg[i][k4] = zero8();
+        vreg[i][k4] = zero8();
+        if (u < QUADS && key >= key_lo && key <= key_hi) {
+          const size_t off = ((size_t)slot(key) * Hkv + kvh) * D + dc * 8;
+          kreg[i][k4] = *reinterpret_cast<const bf16x8*>(k_cache + off);
+          vreg[i][k4] = *reinterpret_cast<const bf16x8*>(v_cache + off);
+        }
+      }
+    }
+  };
+  auto stash = [&]() {                                     // registers -> LDS: K as it is, V transposed
+#pragma unroll
+    for (int i = 0; i < QPT; ++i) {
+      const int u = tid + i * 256;
+      if (u < QUADS) {
+        const int kq = u / CH, dc = u % CH;
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) *reinterpret_cast<bf16x8*>(k_s + (kq * 4 + k4) * KPITCH + dc * 8) = kreg[i][k4];
+        const int vcol = (kq * 4) ^ ((dc & SWZ_MASK) << 2);  // (d >> 3) is dc for all eight entries of the piece
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          bf16x4 four;
+#pragma unroll
+          for (int k4 = 0; k4 < 4; ++k4) four[k4] = vreg[i][k4][e];
+          *reinterpret_cast<bf16x4*>(vt_s + (dc * 8 + e) * VPITCH + vcol) = four;
+        }
+      }
+    }
+  };
+
+  if (D % 32 != 0) {                                       // the padded half step of the first product reads zeros
+    for (int c = tid; c < BN * 2; c += 256) *reinterpret_cast<bf16x8*>(k_s + (c / 2) * KPITCH + D + (c % 2) * 8) = zero8();
+  }
+  const int kb0 = (key_lo / BN) * BN;
+  fetch(kb0);
+  for (int kb = kb0; kb <= key_hi; kb += BN) {
+    __syncthreads();                                       // the last tile has been read by every wave
+    stash();
+    __syncthreads();
+    if (kb + BN <= key_hi) fetch(kb + BN);                 // in flight while this tile is computed
+    if (!live || kb > wave_hi) continue;                   // a whole-wave decision; the wave still meets the barriers
     // ---- scores of 64 keys for this wave's 16 rows
     floatx4 s4[KT];
 #pragma unroll
@@ -136,61 +214,77 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
         s4[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[s], s4[kt], 0, 0, 0);
       }
     }
+    // tiles wholly inside every row's range need no mask
+    const bool need_mask = kb + BN - 1 > wave_lo_pos || kb < wave_max_lo;
     float m_tile = -INFINITY;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int key = kb + kt * 16 + grp * 4 + j;
-        const float v = (key <= row_pos && key >= row_lo) ? s4[kt][j] * scale : -INFINITY;
+        float v = s4[kt][j] * scale_log2e;
+        if (need_mask) {
+          const int key = kb + kt * 16 + grp * 4 + j;
+          if (key > row_pos || key < row_lo) v = -INFINITY;
+        }
         s4[kt][j] = v;
         m_tile = fmaxf(m_tile, v);
       }
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-    const float m_new = fmaxf(m_run, m_tile);
+    // The running maximum is only a reference point: as long as no row of the wave has grown by more than 2^6
+    // over its reference, the reference stays and the output needs no rescaling (P stays below 64).
+    const bool grow = __any(m_tile > m_run + 6.0f);
+    const float m_new = grow ? fmaxf(m_run, m_tile) : m_run;
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
-    const float alpha = expf(m_run - m_safe);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
     float psum = 0.f;
-    bf16x4 pa[KT];
+    bf16x8 pa[KT / 2];                                     // P of keys (32 a + 4 grp + j) and (32 a + 16 + 4 grp + j)
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float p = expf(s4[kt][j] - m_safe);
+        const float p = __builtin_amdgcn_exp2f(s4[kt][j] - m_safe);
         psum += p;
-        pa[kt][j] = (__bf16)p;
+        pa[kt / 2][(kt % 2) * 4 + j] = (__bf16)p;
       }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
-    l_run = l_run * alpha + psum;
+    l_part = l_part * alpha + psum;
     m_run = m_new;
-    // rows of the output tiles are 4 grp + j: fetch their factors from the lanes that own those rows
-    float a4[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) a4[j] = __shfl(alpha, grp * 4 + j, 64);
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
+      const int drow = dt * 16 + col;                      // the V^T row this lane reads as operand
+      const int swz = ((drow >> 3) & SWZ_MASK) << 2;
+      if (grow) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o[dt][j] *= a4[j];
+        for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
+      }
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt) {
-        const bf16x4 vb = *reinterpret_cast<const bf16x4*>(vt_s + (dt * 16 + col) * VPITCH + kt * 16 + grp * 4);
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa[kt], vb, o[dt], 0, 0, 0);
+      for (int a = 0; a < KT / 2; ++a) {
+        // this lane's eight summation slots: keys 32 a + 4 grp + (0..3) and 32 a + 16 + 4 grp + (0..3)
+        const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vt_s + drow * VPITCH + ((a * 32 + grp * 4) ^ swz));
+        const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vt_s + drow * VPITCH + ((a * 32 + 16 + grp * 4) ^ swz));
+        bf16x8 va;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          va[j] = lo4[j];
+          va[4 + j] = hi4[j];
+        }
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pa[a], o[dt], 0, 0, 0);
       }
     }
   }
-  if (!wave_live) return;
-  float inv4[4];
+  if (!live) return;
+  float l = l_part;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (row_ok) {
+    const float inv = 1.0f / l;
+    bf16_t* dst = out + ((size_t)(q_begin + row_tok) * Hq + head) * D;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) inv4[j] = 1.0f / __shfl(l_run, grp * 4 + j, 64);
+    for (int dt = 0; dt < DTILES; ++dt) {
+      bf16x4 four;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int tok = tok0 + grp * 4 + j;
-    if (tok < q_len) {
-      bf16_t* dst = out + ((size_t)(q_begin + tok) * Hq + head) * D;
-#pragma unroll
-      for (int dt = 0; dt < DTILES; ++dt) dst[dt * 16 + col] = (bf16_t)(o[dt][j] * inv4[j]);
+      for (int j = 0; j < 4; ++j) four[j] = (__bf16)(o[dt][j] * inv);
+      *reinterpret_cast<bf16x4*>(dst + dt * 16 + grp * 4) = four;
     }
   }
 }
@@ -205,14 +299,23 @@ extern "C" int nhv_prefill_attention_bf16(const void* q, const void* k_cache, co
   NHV_REQUIRE(Hq % Hkv == 0, "prefill attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   NHV_REQUIRE(window >= 0, "prefill attention: negative window");
   NHV_REQUIRE(prefill::SUPPORTED, "prefill attention: head size %d is beyond this kernel's limit of 256", prefill::D);
+  int page_shift = -1;
+  for (int b = 0; b < 31; ++b)
+    if (page_size == (1 << b)) page_shift = b;
   const int G = Hq / Hkv;
   const long long row_tiles = (long long)G * ((max_q_len + 15) / 16);
-  const long long gx = (row_tiles + 3) / 4;
+  const long long gx = (row_tiles + prefill::TPB - 1) / prefill::TPB;
   NHV_REQUIRE(gx <= 0x7fffffff && Hkv <= 65535 && B <= 65535, "prefill attention: grid too large");
-  hipLaunchKernelGGL(prefill::prefill_attention_kernel, dim3((unsigned)gx, Hkv, B), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out,
-                     (const int*)cu_seqlens_q, (const int*)context_lens, (const int*)block_tables, max_blocks, Hq, Hkv,
-                     page_size, scale, window);
+  if (max_blocks <= prefill::BT_LDS)
+    hipLaunchKernelGGL(prefill::prefill_attention_kernel<true>, dim3((unsigned)gx, Hkv, B), dim3(256), 0,
+                       (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out,
+                       (const int*)cu_seqlens_q, (const int*)context_lens, (const int*)block_tables, max_blocks, Hq, Hkv,
+                       page_size, page_shift, scale * 1.4426950408889634f, window);
+  else
+    hipLaunchKernelGGL(prefill::prefill_attention_kernel<false>, dim3((unsigned)gx, Hkv, B), dim3(256), 0,
+                       (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out,
+                       (const int*)cu_seqlens_q, (const int*)context_lens, (const int*)block_tables, max_blocks, Hq, Hkv,
+                       page_size, page_shift, scale * 1.4426950408889634f, window);
   NHV_LAUNCH_CHECK("prefill_attention");
   return 0;
 }

@@ -192,8 +192,36 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   }
 }
 
+// the same, eight entries a thread (widths that are a multiple of 8)
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total8) {
+  const int per_row = I / 8;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / per_row, c = idx % per_row;
+    float g[8], u[8], o[8];
+    load8f<T>(gu + t * 2 * I + c * 8, g);
+    load8f<T>(gu + t * 2 * I + I + c * 8, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = g[e] / (1.0f + expf(-g[e])) * u[e];
+    store8f<T>(out + t * I + c * 8, o);
+  }
+}
+
 extern "C" int nhv_silu_mul(const void* gu, void* out, int T, int I, int dtype, void* stream) {
   NHV_REQUIRE(T > 0 && I > 0, "silu_mul: bad sizes T=%d I=%d", T, I);
+  if (I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const size_t total8 = (size_t)T * (I / 8);
+    const int vblocks = (int)((total8 + 255) / 256 > 65535 * 16 ? 65535 * 16 : (total8 + 255) / 256);
+    hipStream_t vs = (hipStream_t)stream;
+    if (dtype == NHV_F32)
+      hipLaunchKernelGGL(silu_mul_vec_kernel<float>, dim3(vblocks), dim3(256), 0, vs, (const float*)gu, (float*)out, I, total8);
+    else if (dtype == NHV_BF16)
+      hipLaunchKernelGGL(silu_mul_vec_kernel<bf16_t>, dim3(vblocks), dim3(256), 0, vs, (const bf16_t*)gu, (bf16_t*)out, I, total8);
+    else
+      return nhv_fail("silu_mul: unknown dtype %d", dtype);
+    NHV_LAUNCH_CHECK("silu_mul");
+    return 0;
+  }
   const size_t total = (size_t)T * I;
   const int blocks = (int)((total + 255) / 256 > 65535 * 4 ? 65535 * 4 : (total + 255) / 256);
   hipStream_t s = (hipStream_t)stream;
@@ -301,6 +329,76 @@ __global__ void qk_rope_write_kernel(const T* __restrict__ qkv, const T* __restr
   }
 }
 
+// The same for head sizes that are a power of two (and full or no rotation): CH = D / 8 lanes own a head, eight
+// consecutive entries each; the norm's sum and the rotation's partner (entry d +- D/2) come by lane shuffles, nothing
+// goes through LDS, and a wave works on 64 / CH heads at once.
+template <typename T, typename W, int CH>
+__global__ __launch_bounds__(256) void qk_rope_write_vec_kernel(
+    const T* __restrict__ qkv, const T* __restrict__ bias, const W* __restrict__ q_norm_w, const W* __restrict__ k_norm_w,
+    float eps, const float* __restrict__ cos_sin, int rot, const int* __restrict__ positions,
+    const int* __restrict__ slot_mapping, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int Hq,
+    int Hkv, int heads_per_token, long long n_items) {
+  constexpr int D = CH * 8;
+  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long item = gid / CH;
+  const int c = (int)(gid % CH);
+  if (item >= n_items) return;                       // whole heads leave together
+  const int t = (int)(item / heads_per_token), h = (int)(item % heads_per_token);
+  const int width = (Hq + 2 * Hkv) * D;
+  const bool is_q = h < Hq;
+  const bool is_k = !is_q && h < Hq + Hkv;
+  int slot = -1;
+  if (!is_q) {
+    slot = slot_mapping[t];
+    if (slot < 0) return;
+  }
+  float v[8];
+  load8f<T>(qkv + (size_t)t * width + (size_t)h * D + c * 8, v);
+  if (bias) {
+    float b[8];
+    load8f<T>(bias + (size_t)h * D + c * 8, b);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = to_f32(from_f32<T>(v[e] + b[e]));
+  }
+  if (!is_q && !is_k) {
+    store8f<T>(v_cache + ((size_t)slot * Hkv + (h - Hq - Hkv)) * D + c * 8, v);
+    return;
+  }
+  const W* nw = is_q ? q_norm_w : k_norm_w;
+  if (nw) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+#pragma unroll
+    for (int off = 1; off < CH; off <<= 1) ss += __shfl_xor(ss, off, NHV_WAVE);
+    const float r = 1.0f / sqrtf(ss / (float)D + eps);
+    float wv[8];
+    load8f<W>(nw + c * 8, wv);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = to_f32(from_f32<T>(to_f32(from_f32<T>(v[e] * r)) * wv[e]));
+  }
+  float o[8];
+  if (rot > 0) {
+    constexpr int HALF_LANES = CH / 2 > 0 ? CH / 2 : 1;
+    float cs[8], sn[8];
+    const float* row = cos_sin + (size_t)positions[t] * rot;
+    const int j = (c % HALF_LANES) * 8;              // index into the table's cosines; sines lie rot / 2 further
+    load8f<float>(row + j, cs);
+    load8f<float>(row + rot / 2 + j, sn);
+    const bool first_half = c < HALF_LANES;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float partner = __shfl_xor(v[e], HALF_LANES, NHV_WAVE);
+      o[e] = first_half ? v[e] * cs[e] - partner * sn[e] : v[e] * cs[e] + partner * sn[e];
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = v[e];
+  }
+  T* dst = is_q ? q_out + ((size_t)t * Hq + h) * D : k_cache + ((size_t)slot * Hkv + (h - Hq)) * D;
+  store8f<T>(dst + c * 8, o);
+}
+
 extern "C" int nhv_qk_rope_write(const void* qkv, const void* bias, const void* q_norm_w, const void* k_norm_w, float eps,
                                  const void* cos_sin, int rot, int max_pos, const void* positions,
                                  const void* slot_mapping, void* q_out, void* k_cache, void* v_cache, int T, int Hq,
@@ -314,6 +412,39 @@ extern "C" int nhv_qk_rope_write(const void* qkv, const void* bias, const void* 
   const int heads = write_kv ? Hq + 2 * Hkv : Hq;
   const size_t lds = (size_t)D * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
+  // power-of-two head sizes from 16 to 512 with full (or no) rotation: the shuffle kernel
+  const int ch = D / 8;
+  const bool pow2 = D % 8 == 0 && ch >= 2 && ch <= 64 && (ch & (ch - 1)) == 0;
+  const bool aligned = (uintptr_t)qkv % 16 == 0 && (uintptr_t)q_out % 16 == 0 && (uintptr_t)k_cache % 16 == 0 &&
+                       (uintptr_t)v_cache % 16 == 0 && (uintptr_t)bias % 16 == 0 && (uintptr_t)q_norm_w % 16 == 0 &&
+                       (uintptr_t)k_norm_w % 16 == 0 && (uintptr_t)cos_sin % 16 == 0;
+  if (pow2 && aligned && (rot == D || rot == 0)) {
+    const long long n_items = (long long)T * heads;
+    const long long vblocks = (n_items * ch + 255) / 256;
+    NHV_REQUIRE(vblocks <= 0x7fffffff, "qk_rope_write: too many tokens");
+#define VLAUNCH(TT, WW, CHN)                                                                                         \
+  hipLaunchKernelGGL((qk_rope_write_vec_kernel<TT, WW, CHN>), dim3((unsigned)vblocks), dim3(256), 0, s, (const TT*)qkv, \
+                     (const TT*)bias, (const WW*)q_norm_w, (const WW*)k_norm_w, eps, (const float*)cos_sin, rot,     \
+                     (const int*)positions, (const int*)slot_mapping, (TT*)q_out, (TT*)k_cache, (TT*)v_cache, Hq, Hkv, \
+                     heads, n_items)
+#define VBY_CH(TT, WW)                      \
+  switch (ch) {                             \
+    case 2: VLAUNCH(TT, WW, 2); break;      \
+    case 4: VLAUNCH(TT, WW, 4); break;      \
+    case 8: VLAUNCH(TT, WW, 8); break;      \
+    case 16: VLAUNCH(TT, WW, 16); break;    \
+    case 32: VLAUNCH(TT, WW, 32); break;    \
+    default: VLAUNCH(TT, WW, 64); break;    \
+  }
+    if (dtype == NHV_F32 && w_dtype == NHV_F32) { VBY_CH(float, float) }
+    else if (dtype == NHV_BF16 && w_dtype == NHV_BF16) { VBY_CH(bf16_t, bf16_t) }
+    else if (dtype == NHV_BF16 && w_dtype == NHV_F32) { VBY_CH(bf16_t, float) }
+    else return nhv_fail("qk_rope_write: unsupported dtypes x=%d w=%d", dtype, w_dtype);
+#undef VBY_CH
+#undef VLAUNCH
+    NHV_LAUNCH_CHECK("qk_rope_write");
+    return 0;
+  }
 #define LAUNCH(TT, WW)                                                                                              \
   hipLaunchKernelGGL((qk_rope_write_kernel<TT, WW>), dim3((unsigned)((size_t)T * heads)), dim3(NHV_WAVE), lds, s,  \
                      (const TT*)qkv, (const TT*)bias, (const WW*)q_norm_w, (const WW*)k_norm_w, eps,               \
