@@ -29,7 +29,14 @@ TINY_C = {
     "head_dim": 48, "intermediate_size": 112, "vocab_size": 301, "rope_theta": 50000.0, "rms_norm_eps": 1e-5,
     "tie_word_embeddings": False, "max_position_embeddings": 384, "attention_bias": True, "hidden_act": "silu",
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# the head size and group size of the real family (128, 4 query heads per key/value head), otherwise small
+SMALL_D = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "num_hidden_layers": 2, "hidden_size": 512, "num_attention_heads": 8, "num_key_value_heads": 2,
+    "head_dim": 128, "intermediate_size": 1536, "vocab_size": 2048, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "max_position_embeddings": 1024, "attention_bias": False, "hidden_act": "silu",
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (SMALL_D, 3)}
 
 
 def pytest_configure(config):
