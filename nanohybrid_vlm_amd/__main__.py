@@ -90,7 +90,15 @@ def cmd_generate(args) -> int:
 def cmd_bench(args) -> int:
     import torch
     from . import SamplingParams
+    if args.kernel_times and args.mode != "eager":
+        print("--kernel-times needs --mode eager", file=sys.stderr)
+        return 2
     llm = _make_llm(args)
+    timer = None
+    if args.kernel_times:
+        from .native import ops
+        timer = ops.kernel_times()
+        times = timer.__enter__()
     vocab = llm.runner.vocab_size
     gen = torch.Generator().manual_seed(args.seed)
     results = []
@@ -131,6 +139,10 @@ def cmd_bench(args) -> int:
                 "preemptions": llm.scheduler.num_preemptions,
             })
             print(json.dumps(results[-1]), flush=True)
+    if timer is not None:
+        timer.__exit__(None, None, None)
+        print(times.table())
+    print(json.dumps({"memory": llm.get_memory_stats()}), flush=True)
     if args.output:
         Path(args.output).write_text(json.dumps({"model": args.model, "mode": args.mode, "dtype": args.dtype,
                                                  "token_budget": args.token_budget, "results": results}, indent=2))
@@ -185,6 +197,8 @@ def main(argv=None) -> int:
     b.add_argument("--repeats", type=int, default=2)
     b.add_argument("--warmup-output-tokens", type=int, default=8)
     b.add_argument("--label", default="run")
+    b.add_argument("--kernel-times", action="store_true",
+                   help="print the device time per kernel (eager mode only: events around every kernel call)")
     b.add_argument("--output", help="JSON file for all results")
     b.set_defaults(fn=cmd_bench)
 

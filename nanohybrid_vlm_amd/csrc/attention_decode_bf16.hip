@@ -2,17 +2,20 @@
 // Compiled for one head size: -DNHV_HEAD_DIM=<multiple of 16>.
 //
 // One wave works on (token, key/value head, split of the keys). The G query heads
-// that share the key/value head (G <= 16) are the 16 columns of an MFMA tile:
-//   S^T[key, head] = K[key, :] . Q[head, :]   v_mfma_f32_16x16x32_bf16, K rows straight from the cache
-// so every lane ends up with four consecutive keys of one head and the running
-// maximum needs two shuffles. The probabilities go through LDS to the second half,
-// which is plain FMA work: with one token per request the values are read once and
-// used by only G heads, so the step is bound by the cache's bandwidth, not by math.
-//   O[head, d] += P[head, key] * V[key, d]    lanes own 8 consecutive d of every 64/LPK-th key
-// Splits are aligned to absolute key positions. Each split writes its unnormalised
-// output with (maximum, sum) in float; a second kernel merges the splits in rising
-// order. Keys that are not visible are loaded as zeros (the cache's unused slots
-// may hold anything).
+// that share the key/value head (G <= 16) are the 16 columns of the MFMA tiles:
+//   S^T[key, head]  = K[key, :] . Q[head, :]        K rows straight from the cache (v_mfma_f32_16x16x32_bf16)
+//   running maximum per head in float (two shuffles), sums kept per lane
+//   O^T[d, head]   += V^T[d, key] . P^T[key, head]   V^T from the wave's own LDS tile, P in registers
+// Keys are taken 32 a round; all keys and values of a round are asked for from memory
+// before anything is computed. The values are written to LDS transposed (four keys,
+// 8 bytes, at a time, columns XOR-ed against bank conflicts), which turns the second
+// half from 64 x G x D multiply-adds on the vector lanes into 16 matrix instructions.
+// The S^T tiles leave every lane with keys of one head in the order in which the second
+// product sums them, so P never leaves the registers, and a lane's outputs belong to
+// the head of its scores: rescaling needs no exchange. Splits are aligned to absolute
+// key positions. Each split writes its unnormalised output with (maximum, sum) in
+// float; a second kernel merges the splits in rising order. Keys that are not visible
+// are loaded as zeros (the cache's unused slots may hold anything).
 #include "nhv_common.h"
 #include <math.h>
 
@@ -21,16 +24,21 @@
 #endif
 
 constexpr int D = NHV_HEAD_DIM;
-static_assert(D % 16 == 0 && D >= 16 && D <= 512, "head size must be a multiple of 16 up to 512");
-constexpr int DSTEPS = (D + 31) / 32;                       // MFMA steps over the head
+static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
+constexpr int DSTEPS = (D + 31) / 32;                       // MFMA steps over the head in the first product
+constexpr int DTILES = D / 16;                              // output tiles of the second product
 constexpr int CHUNKS = D / 8;                               // 16-byte pieces of a row
-constexpr int LPK = CHUNKS <= 2 ? 2 : CHUNKS <= 4 ? 4 : CHUNKS <= 8 ? 8 : CHUNKS <= 16 ? 16 : CHUNKS <= 32 ? 32 : 64;
-constexpr int KPP = 64 / LPK;                               // keys per pass of the value half
-constexpr int RK = 64;                                      // keys per round
+constexpr int LPK = CHUNKS <= 2 ? 2 : CHUNKS <= 4 ? 4 : CHUNKS <= 8 ? 8 : CHUNKS <= 16 ? 16 : 32;   // lanes per key
+constexpr int KPP = 64 / LPK;                               // keys per load instruction of the values
+constexpr int RK = 32;                                      // keys per round (64 needs 238 registers: one wave per SIMD)
 constexpr int KT = RK / 16;                                 // MFMA tiles of 16 keys per round
-constexpr int PASSES = RK / KPP;                            // passes of the value half per round
+constexpr int PASSES = RK / KPP;                            // value loads per lane and round: consecutive keys
+constexpr int KG = PASSES >= 4 ? 4 : PASSES;                // keys per transposed LDS write
+constexpr int VPITCH = RK + 8;                              // elements per row of the V^T tile
+constexpr int SWZ_MASK = RK / 4 - 1;
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
@@ -47,14 +55,12 @@ __device__ __forceinline__ int slot_of(const int* bt, int key, int page_size, in
   return bt[key / page_size] * page_size + key % page_size;
 }
 
-template <int GC>
 __global__ __launch_bounds__(64) void decode_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     float* __restrict__ part_o, float* __restrict__ part_ml, const int* __restrict__ token_req,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv,
-    int page_size, int page_shift, float scale, int window, int split_len, int n_splits) {
-  __shared__ __attribute__((aligned(16))) float p_s[RK][20];          // [key][head], rows of 16-byte pieces
-  __shared__ float alpha_s[16];
+    int page_size, int page_shift, float scale_log2e, int window, int split_len, int n_splits) {
+  __shared__ __attribute__((aligned(16))) bf16_t vt_s[D * VPITCH];
   const int lane = threadIdx.x;
   const int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
   const int G = Hq / Hkv;
@@ -74,17 +80,15 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
     qb[s] = (col < G && d < D) ? load8(q + ((size_t)t * Hq + kvh * G + col) * D + d) : zero8();
   }
 
-  float m_run = -INFINITY, l_part = 0.f;     // per head `col`; l_part is this lane's share of the sum
-  float acc[GC][8];
+  float m_run = -INFINITY, l_part = 0.f;     // of head `col` (base 2); l_part is this lane's share of the sum
+  floatx4 o[DTILES];                          // o[dt][j]: entry dt * 16 + 4 grp + j of head `col`
 #pragma unroll
-  for (int g = 0; g < GC; ++g)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
-  const int ksub = lane / LPK, chunk = lane % LPK;
+  for (int dt = 0; dt < DTILES; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int ksub = lane / LPK, chunk = lane % LPK;       // this lane loads piece `chunk` of keys ksub * PASSES + (0..PASSES)
   const bool chunk_live = chunk * 8 < D;
 
   for (int kb = (first / RK) * RK; kb <= last; kb += RK) {
-    // ---- all keys and values of the round are asked for before anything is computed: 64 keys, 32 KB a wave
+    // ---- all keys and values of the round are asked for before anything is computed (16 KB a wave at head size 128)
     // (pages that are a power of two of at least 64 tokens hold a whole round: one look at the block table)
     const bool one_page = page_shift >= 6;
     const int round_base = one_page ? (bt[kb >> page_shift] << page_shift) : 0;
@@ -105,7 +109,7 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
     bf16x8 vv[PASSES];
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-      const int key = kb + ps * KPP + ksub;
+      const int key = kb + ksub * PASSES + ps;
       const bool ok = chunk_live && key >= first && key <= last;
       int slot = 0;
       if (ok) slot = one_page ? round_base + (key & (page_size - 1)) : slot_of(bt, key, page_size, page_shift);
@@ -119,6 +123,28 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
 #pragma unroll
       for (int s = 0; s < DSTEPS; ++s) s4[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kt][s], qb[s], s4[kt], 0, 0, 0);
     }
+    // ---- values into LDS, transposed: row d, columns = keys of the round
+    __syncthreads();                                   // the last round's tile has been read
+    if (chunk_live) {
+#pragma unroll
+      for (int pg = 0; pg < PASSES / KG; ++pg) {
+        const int key0 = ksub * PASSES + pg * KG;      // KG consecutive keys of this lane
+        const int vcol = key0 ^ ((chunk & SWZ_MASK) << 2);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          bf16_t* dst = vt_s + (chunk * 8 + e) * VPITCH + vcol;
+          if (KG == 4) {
+            bf16x4 four;
+#pragma unroll
+            for (int k4 = 0; k4 < 4; ++k4) four[k4] = vv[pg * KG + k4][e];
+            *reinterpret_cast<bf16x4*>(dst) = four;
+          } else {
+#pragma unroll
+            for (int k4 = 0; k4 < KG; ++k4) dst[k4] = vv[pg * KG + k4][e];
+          }
+        }
+      }
+    }
     // ---- running softmax for head `col` over keys kb + 16 kt + 4 grp + j
     float m_tile = -INFINITY;
 #pragma unroll
@@ -126,82 +152,64 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int key = kb + kt * 16 + grp * 4 + j;
-        const float v = (key >= first && key <= last) ? s4[kt][j] * scale : -INFINITY;
+        const float v = (key >= first && key <= last) ? s4[kt][j] * scale_log2e : -INFINITY;
         s4[kt][j] = v;
         m_tile = fmaxf(m_tile, v);
       }
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-    const float m_new = fmaxf(m_run, m_tile);          // finite: every round holds a visible key
-    const float alpha = __expf(m_run - m_new);
+    // the maximum is a reference point only: it moves when some head has grown by more than 2^6 over it
+    const bool grow = __any(m_tile > m_run + 6.0f);
+    const float m_new = grow ? fmaxf(m_run, m_tile) : m_run;     // finite: every round holds a visible key
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float psum = 0.f;
-    __syncthreads();                                   // the last round's p_s and alpha_s have been read
+    bf16x8 pa[KT / 2];                                 // P of keys (32 a + 4 grp + j) and (32 a + 16 + 4 grp + j)
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float p = __expf(s4[kt][j] - m_new);     // exp(-inf) = 0 for keys out of range
-        p_s[kt * 16 + grp * 4 + j][col] = p;
+        const float p = __builtin_amdgcn_exp2f(s4[kt][j] - m_new);   // 0 for keys out of range
         psum += p;
+        pa[kt / 2][(kt % 2) * 4 + j] = (__bf16)p;
       }
     l_part = l_part * alpha + psum;
     m_run = m_new;
-    if (grp == 0) alpha_s[col] = alpha;
-    __syncthreads();
-    // ---- O += P V
+    __syncthreads();                                   // the tile is written
+    // ---- O^T += V^T P^T
 #pragma unroll
-    for (int g = 0; g < GC; ++g) {
-      const float a = alpha_s[g];
+    for (int dt = 0; dt < DTILES; ++dt) {
+      const int drow = dt * 16 + col;
+      const int swz = ((drow >> 3) & SWZ_MASK) << 2;
+      if (grow) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[g][e] *= a;
-    }
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-      const int kl = ps * KPP + ksub;
-      float vf[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) vf[e] = (float)vv[ps][e];
-      float pg[GC];
-      if (GC >= 4) {
-#pragma unroll
-        for (int g4 = 0; g4 < GC / 4; ++g4) {
-          const float4 p4 = *reinterpret_cast<const float4*>(&p_s[kl][g4 * 4]);
-          pg[g4 * 4] = p4.x; pg[g4 * 4 + 1] = p4.y; pg[g4 * 4 + 2] = p4.z; pg[g4 * 4 + 3] = p4.w;
-        }
-      } else {
-#pragma unroll
-        for (int g = 0; g < GC; ++g) pg[g] = p_s[kl][g];
+        for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
       }
 #pragma unroll
-      for (int g = 0; g < GC; ++g)
+      for (int a = 0; a < KT / 2; ++a) {
+        const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vt_s + drow * VPITCH + ((a * 32 + grp * 4) ^ swz));
+        const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vt_s + drow * VPITCH + ((a * 32 + 16 + grp * 4) ^ swz));
+        bf16x8 va;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pg[g], vf[e], acc[g][e]);
+        for (int j = 0; j < 4; ++j) {
+          va[j] = lo4[j];
+          va[4 + j] = hi4[j];
+        }
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pa[a], o[dt], 0, 0, 0);
+      }
     }
   }
-  // ---- this split's result: sum over the lanes that hold other keys of the same chunk
-#pragma unroll
-  for (int off = LPK; off < 64; off <<= 1) {
-#pragma unroll
-    for (int g = 0; g < GC; ++g)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[g][e] += __shfl_xor(acc[g][e], off, 64);
-  }
+  // ---- this split's result
   l_part += __shfl_xor(l_part, 16, 64);
   l_part += __shfl_xor(l_part, 32, 64);
-  if (lane < 16 && lane < G) {
-    float* ml = part_ml + (((size_t)t * Hq + kvh * G + lane) * n_splits + split) * 2;
-    ml[0] = m_run;
-    ml[1] = l_part;
-  }
-  if (ksub == 0 && chunk_live) {
-#pragma unroll
-    for (int g = 0; g < GC; ++g) {
-      if (g < G) {
-        float* o = part_o + (((size_t)t * Hq + kvh * G + g) * n_splits + split) * D + chunk * 8;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = acc[g][e];
-      }
+  if (col < G) {
+    const size_t item = ((size_t)t * Hq + kvh * G + col) * n_splits + split;
+    if (grp == 0) {
+      part_ml[item * 2] = m_run;
+      part_ml[item * 2 + 1] = l_part;
     }
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+      *reinterpret_cast<float4*>(part_o + item * D + dt * 16 + grp * 4) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
   }
 }
 
@@ -227,7 +235,7 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
   for (int s = s0 + lane; s <= s1; s += 64) m = fmaxf(m, ml[s * 2]);
   m = wave_max(m);
   float l = 0.f;
-  for (int s = s0 + lane; s <= s1; s += 64) l += ml[s * 2 + 1] * expf(ml[s * 2] - m);
+  for (int s = s0 + lane; s <= s1; s += 64) l += ml[s * 2 + 1] * exp2f(ml[s * 2] - m);
   l = wave_sum(l);
   const float inv = 1.0f / l;
   const float* po = part_o + (size_t)item * n_splits * D;
@@ -237,7 +245,7 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
   for (int i = 0; i < MPIECES; ++i) acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 4
   for (int s = s0 + sub; s <= s1; s += MROWS) {
-    const float wgt = expf(ml[s * 2] - m);
+    const float wgt = exp2f(ml[s * 2] - m);
 #pragma unroll
     for (int i = 0; i < MPIECES; ++i) {
       const int qd = piece + i * MLPR;
@@ -288,17 +296,10 @@ extern "C" int nhv_decode_attention_bf16(const void* q, const void* k_cache, con
   NHV_REQUIRE(window >= 0, "decode attention: negative window");
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(n_splits, Hkv, T);
-#define LAUNCH(GC)                                                                                                    \
-  hipLaunchKernelGGL(decode_attention_kernel<GC>, grid, dim3(64), 0, s, (const bf16_t*)q, (const bf16_t*)k_cache,     \
-                     (const bf16_t*)v_cache, (float*)part_o, (float*)part_ml, (const int*)token_req,                  \
-                     (const int*)positions, (const int*)block_tables, max_blocks, Hq, Hkv, page_size, page_shift, scale,   \
-                     window, split_len, n_splits)
-  if (G <= 1) LAUNCH(1);
-  else if (G <= 2) LAUNCH(2);
-  else if (G <= 4) LAUNCH(4);
-  else if (G <= 8) LAUNCH(8);
-  else LAUNCH(16);
-#undef LAUNCH
+  hipLaunchKernelGGL(decode_attention_kernel, grid, dim3(64), 0, s, (const bf16_t*)q, (const bf16_t*)k_cache,
+                     (const bf16_t*)v_cache, (float*)part_o, (float*)part_ml, (const int*)token_req,
+                     (const int*)positions, (const int*)block_tables, max_blocks, Hq, Hkv, page_size, page_shift,
+                     scale * 1.4426950408889634f, window, split_len, n_splits);
   NHV_LAUNCH_CHECK("decode_attention");
   hipLaunchKernelGGL(merge_splits_kernel, dim3((unsigned)((size_t)T * Hq)), dim3(64), 0, s, (const float*)part_o,
                      (const float*)part_ml, (bf16_t*)out, (const int*)positions, window, split_len, n_splits, Hq);

@@ -229,6 +229,9 @@ class LLM:
             result.append({"text": text, "token_ids": token_ids})
         return result
 
+    def get_memory_stats(self) -> dict:
+        return self.runner.get_memory_stats()
+
     def get_completed_request_metrics(self) -> list[RequestMetrics]:
         out, self._completed_metrics = self._completed_metrics, []
         return out

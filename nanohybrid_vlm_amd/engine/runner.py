@@ -349,6 +349,32 @@ class ModelRunner:
             backend.own_kernels_only = old
         return {"graph": graph, "index": index, "logits": logits, "ctx": ctx}
 
+    def get_memory_stats(self) -> dict:
+        """Bytes of weights, cache and state pools, pages per group, and the allocator's and the device's view
+        (nanovllm/engine/model_runner.py:260-371 reports the same kinds of figures)."""
+        params = getattr(self.model, "parameters", {}) or {}
+        seen, weight_bytes = set(), 0
+        for t in params.values():
+            if t.data_ptr() not in seen:                    # a tied head shares the embedding's storage
+                seen.add(t.data_ptr())
+                weight_bytes += t.numel() * t.element_size()
+        stats = {
+            "weight_bytes": weight_bytes,
+            "kv_cache_bytes": sum(t.numel() * t.element_size() for t in self.kv_tensors),
+            "state_pool_bytes": sum(t.numel() * t.element_size() for pool in self.state_pools for t in pool.values()),
+            "page_size": self.page_size,
+            "groups": [{"name": g.name, "window": g.window, "pages": g.num_pages,
+                        "free_pages": self.cache.num_free_pages(i)} for i, g in enumerate(self.cache.groups)],
+            "live_requests": len(self.cache.requests),
+            "graphs_recorded": sorted(self._graphs),
+        }
+        if self.device.type == "cuda":
+            free, total = torch.cuda.mem_get_info(self.device)
+            stats.update(device_free_bytes=free, device_total_bytes=total,
+                         torch_allocated_bytes=torch.cuda.memory_allocated(self.device),
+                         torch_reserved_bytes=torch.cuda.memory_reserved(self.device))
+        return stats
+
     def finish(self, request_id) -> None:
         """The request is over: its pages and its state slot are given back."""
         if request_id in self.cache:

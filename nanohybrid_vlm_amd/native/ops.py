@@ -202,6 +202,52 @@ class NativeBackend:
         self._call("nhv_sample", _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(tokens), n, V, _stream())
 
 
+class KernelTimes:
+    """Per-kernel device time of everything launched inside ``with kernel_times() as t`` (events around every
+    call into the library; not for use while a graph is recorded). ``t.table()`` after the block."""
+
+    def __init__(self):
+        self.records: list[tuple[str, torch.cuda.Event, torch.cuda.Event]] = []
+
+    def summary(self) -> dict[str, tuple[int, float]]:
+        torch.cuda.synchronize()
+        out: dict[str, tuple[int, float]] = {}
+        for name, start, end in self.records:
+            n, ms = out.get(name, (0, 0.0))
+            out[name] = (n + 1, ms + start.elapsed_time(end))
+        return out
+
+    def table(self) -> str:
+        rows = sorted(self.summary().items(), key=lambda kv: -kv[1][1])
+        total = sum(ms for _, (_, ms) in rows) or 1.0
+        lines = [f"{'kernel':40s} {'calls':>7s} {'total ms':>10s} {'mean us':>9s} {'share':>6s}"]
+        for name, (n, ms) in rows:
+            lines.append(f"{name:40s} {n:7d} {ms:10.3f} {ms / n * 1e3:9.1f} {100 * ms / total:5.1f}%")
+        return "\n".join(lines)
+
+
+class kernel_times:
+    def __enter__(self) -> KernelTimes:
+        self.times = KernelTimes()
+        b = backend()
+        self._old = b._call
+        times = self.times
+
+        def timed_call(fn_name, *args, lib=None):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            self._old(fn_name, *args, lib=lib)
+            end.record()
+            times.records.append((fn_name, start, end))
+
+        b._call = timed_call
+        return self.times
+
+    def __exit__(self, *exc):
+        backend()._call = self._old
+        return False
+
+
 _backend = None
 
 

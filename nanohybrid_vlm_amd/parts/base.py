@@ -75,6 +75,8 @@ class Part:
         return out
 
     def bind_all(self, params: dict[str, torch.Tensor], prefix: str = "") -> None:
+        if prefix == "":
+            self.parameters = params            # the whole tree's tensors by name, kept at the root
         own = {k: params[prefix + k] for k in self.param_specs()}
         self.bind(own)
         for cname, child in self.children().items():

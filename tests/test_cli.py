@@ -40,3 +40,7 @@ def test_generate_and_bench_commands(model_folders, tmp_path):
          "--max-model-len", "128", "--label", "tiny", "--mode", "graph", "--output", result)
     data = json.loads(open(result).read())
     assert len(data["results"]) == 2 and all(r["decode_tok_s"] > 0 and r["ttft_ms_mean"] > 0 for r in data["results"])
+    out = _run("bench", "--model", folder, "--cases", "16:2", "--output-tokens", "4", "--repeats", "1", "--block-size", "8",
+               "--num-blocks", "32", "--max-model-len", "64", "--mode", "eager", "--kernel-times")
+    assert "nhv_paged_attention" in out or "nhv_decode_attention_bf16" in out
+    assert "nhv_rmsnorm" in out and '"memory"' in out

@@ -51,6 +51,9 @@ def _run(folder, device, dtype, name, **options):
         assert o["token_ids"] == want, f"temperature, prompt {i}"
     metrics = llm.get_completed_request_metrics()
     assert len(metrics) == 2 * len(prompts) and all(m.ttft_ms >= 0 and m.e2e_ms >= m.ttft_ms for m in metrics)
+    stats = llm.get_memory_stats()
+    assert stats["weight_bytes"] > 0 and stats["kv_cache_bytes"] > 0 and stats["live_requests"] == 0
+    assert stats["groups"][0]["free_pages"] == stats["groups"][0]["pages"]
     return llm
 
 
