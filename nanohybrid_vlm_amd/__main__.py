@@ -35,7 +35,12 @@ def _case(text: str) -> tuple[int, int]:
 
 
 def _engine_options(ap: argparse.ArgumentParser) -> None:
-    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--model", help="folder with config.json and model.safetensors")
+    ap.add_argument("--random-weights", type=int, metavar="SEED",
+                    help="instead of --model: random weights of --shape, drawn on the device")
+    ap.add_argument("--shape", default="tinyA", choices=("tinyA", "tinyB", "8b", "14b", "32b"),
+                    help="sizes of the model for --random-weights")
+    ap.add_argument("--layers", type=int, help="with --random-weights: override num_hidden_layers")
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32", "bf16", "fp32"))
     ap.add_argument("--mode", choices=("eager", "graph"), default="graph", help="graph: decode steps replay HIP graphs")
     ap.add_argument("--token-budget", type=int, default=2048, help="tokens per step (max_num_batched_tokens)")
@@ -46,14 +51,36 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--max-model-len", type=int, default=4096)
     ap.add_argument("--scheduler-policy", choices=("decode_first", "prefill_first"), default="decode_first")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--enable-prefix-cache", action="store_true",
+                    help="requests with a common start share the full pages that hold it")
 
 
 def _make_llm(args):
     from . import LLM
-    return LLM(args.model, dtype=args.dtype, enforce_eager=args.mode == "eager",
+    if (args.model is None) == (args.random_weights is None):
+        raise SystemExit("give either --model DIR or --random-weights SEED")
+    built, label = None, args.model
+    if args.random_weights is not None:
+        import torch
+        from .config.registry import resolve_architecture
+        from .parts.model import DecoderModel
+        from .shapes import SHAPES
+        from .weights.random_init import fill_random_on_device
+        raw = dict(SHAPES[args.shape])
+        if args.layers:
+            raw["num_hidden_layers"] = args.layers
+        arch = resolve_architecture(raw)
+        cfg = arch.parse_config(raw)
+        model = DecoderModel(arch.build_spec(cfg))
+        dtype = torch.bfloat16 if args.dtype in ("bfloat16", "bf16") else torch.float32
+        fill_random_on_device(model, seed=args.random_weights, dtype=dtype, device="cuda:0")
+        built, label = (arch, cfg, model), f"random {args.shape}"
+        args.model = label
+    return LLM(label, built_model=built, dtype=args.dtype, enforce_eager=args.mode == "eager",
                max_num_batched_tokens=args.token_budget, gpu_memory_utilization=args.gpu_memory_utilization,
                kvcache_block_size=args.block_size, num_kvcache_blocks=args.num_blocks, max_num_seqs=args.max_num_seqs,
-               max_model_len=args.max_model_len, scheduler_policy=args.scheduler_policy, seed=args.seed)
+               max_model_len=args.max_model_len, scheduler_policy=args.scheduler_policy, seed=args.seed,
+               enable_prefix_cache=args.enable_prefix_cache)
 
 
 def _percentile(values, q):

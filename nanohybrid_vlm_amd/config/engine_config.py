@@ -27,6 +27,7 @@ class EngineConfig:
     kvcache_block_size: int = 256               # tokens in a page (any positive number)
     num_kvcache_blocks: int = -1                # -1: sized from free memory
     num_state_slots: int = -1                   # -1: max_num_seqs
+    enable_prefix_cache: bool = False           # requests with a common start share its full pages
     dtype: str = "bfloat16"                     # "bfloat16" or "float32" (true 32-bit everywhere)
     seed: int = 0                               # default seed of temperature sampling
     device: str = "cuda:0"                      # the one GPU

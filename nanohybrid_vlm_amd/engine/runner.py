@@ -46,7 +46,8 @@ class ModelRunner:
     def __init__(self, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 256,
                  num_pages: int | None = None, num_state_slots: int = 512, gpu_memory_utilization: float = 0.9,
                  max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None, use_graphs: bool = False,
-                 max_model_len: int | None = None, max_graph_batch: int = 16):
+                 max_model_len: int | None = None, max_graph_batch: int = 16, poison_freed_pages: bool = False,
+                 share_prefixes: bool = False):
         """``model``/``arch``/``cfg`` may be given ready-made (weights already bound)
         instead of being read from ``model_dir``."""
         if dtype not in _TORCH_DTYPES:
@@ -64,9 +65,16 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         self.max_position = model.spec.max_position
         self.page_size = page_size
+        if share_prefixes and poison_freed_pages:
+            raise ValueError("a freed page keeps its content for later requests when prefixes are shared; "
+                             "poison_freed_pages would destroy it")
+        self.share_prefixes = share_prefixes
         self._make_cache(page_size, num_pages, num_state_slots, gpu_memory_utilization, max_num_batched_tokens)
         self._pinned = None
         self._pinned_free = None
+        # a debugging aid: pages that are given back are filled with NaN, so that a read of a page that a
+        # request no longer owns shows up in its logits
+        self.poison_freed_pages = poison_freed_pages
         # decode-only steps replay a HIP graph per batch-size bucket (the reference captures CUDA graphs for
         # the same batch sizes, nanovllm/engine/model_runner.py:2559-2594). Up to 16 requests a step is bound
         # by launches and by the own few-rows kernels; larger batches run eagerly, where the matrix products
@@ -96,7 +104,11 @@ class ModelRunner:
         self.num_pages = num_pages
         groups = [PagedGroupSpec(name="all keys" if w is None else f"window {w}", page_size=page_size,
                                  num_pages=num_pages, window=w) for w in windows]
-        self.cache = CacheManager(groups, num_state_slots)
+        if self.share_prefixes and any(isinstance(n, StateNeed) for n in needs):
+            # state of fixed size summarises all earlier tokens: pages alone do not bring a prefix back
+            # (the reference switches the page hashes off for such models, nanovllm/config.py:384-399)
+            raise ValueError("prefixes cannot be shared by a model with per-request state")
+        self.cache = CacheManager(groups, num_state_slots, share_prefixes=self.share_prefixes)
         views: list[CacheView | None] = [None] * len(needs)
         self.kv_tensors: list[torch.Tensor] = []
         self.state_pools: list[dict] = []
@@ -280,8 +292,17 @@ class ModelRunner:
         hidden = self.model.forward(ctx)
         logits = self.model.logits(hidden) if hidden is not None else None
         for e, n in zip(entries, new_lens):
-            self.cache.commit(e.request_id, n)
+            self._poison(self.cache.commit(e.request_id, n, e.tokens))
         return logits
+
+    def _poison(self, given_back: list[list[int]]) -> None:
+        if not self.poison_freed_pages or not any(given_back):
+            return
+        for view in self.model.cache_views:
+            if view.kind == "paged" and view.writes and given_back[view.group]:
+                pages = torch.tensor(given_back[view.group], device=self.device)
+                view.k[pages] = float("nan")
+                view.v[pages] = float("nan")
 
     # ------------------------------------------------------------------ decode steps as HIP graphs
     def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor | None:
@@ -314,7 +335,7 @@ class ModelRunner:
         self._pinned_free.record()
         g["graph"].replay()
         for e, n in zip(entries, meta["new_lens"]):
-            self.cache.commit(e.request_id, n)
+            self._poison(self.cache.commit(e.request_id, n, e.tokens))
         rows = meta["rows"]
         if not rows:
             return None
@@ -366,6 +387,8 @@ class ModelRunner:
             "groups": [{"name": g.name, "window": g.window, "pages": g.num_pages,
                         "free_pages": self.cache.num_free_pages(i)} for i, g in enumerate(self.cache.groups)],
             "live_requests": len(self.cache.requests),
+            "prefix_cache": {"enabled": self.cache.share_prefixes, "known_pages": len(self.cache.page_of_hash),
+                             "shared_tokens": self.cache.num_shared_tokens},
             "graphs_recorded": sorted(self._graphs),
         }
         if self.device.type == "cuda":
@@ -378,4 +401,4 @@ class ModelRunner:
     def finish(self, request_id) -> None:
         """The request is over: its pages and its state slot are given back."""
         if request_id in self.cache:
-            self.cache.release(request_id)
+            self._poison(self.cache.release(request_id))

@@ -157,8 +157,7 @@ class Scheduler:
             seq = self.waiting[0]
             if seq.seq_id not in self.cache:
                 def resources_available() -> bool:
-                    return (num_active < self.max_num_seqs and self.cache.can_admit()
-                            and self.cache.can_reserve(seq.seq_id, seq.num_tokens))
+                    return num_active < self.max_num_seqs and self.cache.can_start(seq.token_ids)
                 while reserve_prefill and not resources_available():
                     # requests that already have a place in this step stay: the decoding ones and (unlike
                     # the reference, scheduler.py:674-719, which would push them out) the prompts just planned
@@ -174,8 +173,11 @@ class Scheduler:
                     break
                 # pages for the whole request as it stands (prompt, and generated tokens of a request
                 # that is computed again), so that no portion can run out of pages (block_manager.py:696-749)
-                self.cache.admit(seq.seq_id)
+                self.cache.admit(seq.seq_id, seq.token_ids)
                 self.cache.reserve(seq.seq_id, seq.num_tokens)
+                # with shared prefixes the first pages may hold this request's first tokens already
+                # (nanovllm/engine/block_manager.py:727-749)
+                seq.num_cached_tokens = self.cache.num_tokens(seq.seq_id)
                 num_active += 1
             left = seq.num_tokens - seq.num_cached_tokens
             if left <= 0:

@@ -44,3 +44,14 @@ def test_generate_and_bench_commands(model_folders, tmp_path):
                "--num-blocks", "32", "--max-model-len", "64", "--mode", "eager", "--kernel-times")
     assert "nhv_paged_attention" in out or "nhv_decode_attention_bf16" in out
     assert "nhv_rmsnorm" in out and '"memory"' in out
+    # random weights drawn on the device, and the prefix cache switched on
+    out = json.loads(_run("generate", "--random-weights", "4", "--shape", "tinyB", "--prompt-ids", "5 17 3",
+                          "--output-tokens", "4", "--temperature", "0", "--ignore-eos", "--block-size", "8", "--num-blocks",
+                          "16", "--max-model-len", "64", "--enable-prefix-cache", "--quiet"))
+    assert len(out[0]["token_ids"]) == 4
+
+
+def test_model_or_random_weights_is_needed():
+    proc = subprocess.run([sys.executable, "-m", "nanohybrid_vlm_amd", "generate", "--prompt-ids", "1"], cwd=REPO,
+                          capture_output=True, text=True, timeout=120)
+    assert proc.returncode != 0 and "--model DIR or --random-weights SEED" in proc.stderr

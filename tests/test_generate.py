@@ -97,6 +97,45 @@ def test_generate_bfloat16_on_gpu(model_folders, name):
             ids.append(t)
 
 
+def _shared_start_run(folder, device, dtype, name, **options):
+    """Prompts with the same first tokens, in a cache so small that requests are pushed out and come back: with
+    the prefix cache on, the tokens are those of the plain implementation and fewer of them are computed."""
+    cfg, w = plain.read_model_folder(folder)
+    start = random_tokens(cfg["vocab_size"], 21, 7)
+    prompts = [start + random_tokens(cfg["vocab_size"], n, 70 + n) for n in (1, 6, 12, 3)] + [start[:17]]
+    greedy = SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True)
+    # a budget of 24 tokens a step: the first prompt and the start of the second run before any page is known
+    llm = LLM(folder, device=device, dtype=dtype, enable_prefix_cache=True, kvcache_block_size=8,
+              max_num_batched_tokens=24, **options)
+    outs = llm.generate(prompts, greedy, use_tqdm=False)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        assert o["token_ids"] == _plain_generate(cfg, w, p, greedy, i, 0, cfg.get("eos_token_id")), f"prompt {i}"
+    llm.runner.cache.check()
+    assert llm.runner.cache.num_shared_tokens >= 16 * (len(prompts) - 2)
+    return llm
+
+
+@pytest.mark.parametrize("options", [dict(num_kvcache_blocks=64), dict(num_kvcache_blocks=11, max_num_seqs=3)])
+def test_prefix_cache_on_emulated_kernels(model_folders, emulated_kernels, options):
+    llm = _shared_start_run(model_folders["B"], "cpu", "float32", "B", **options)
+    if options["num_kvcache_blocks"] == 11:
+        assert llm.scheduler.num_preemptions > 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("options", [dict(num_kvcache_blocks=64), dict(num_kvcache_blocks=11, max_num_seqs=3),
+                                     dict(num_kvcache_blocks=64, enforce_eager=True)])
+def test_prefix_cache_on_gpu(model_folders, options):
+    _shared_start_run(model_folders["B"], "cuda:0", "float32", "B", **options)
+
+
+def test_prefix_cache_refusals(model_folders, emulated_kernels):
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    with pytest.raises(ValueError, match="poison_freed_pages would destroy"):
+        ModelRunner(model_folders["A"], dtype="float32", device="cpu", page_size=4, num_pages=8, num_state_slots=2,
+                    share_prefixes=True, poison_freed_pages=True)
+
+
 def test_late_arrivals_and_step_by_hand(model_folders, emulated_kernels):
     """Requests added while others decode (nanovllm's tests drive llm.step() the same way,
     tests/5090-test-TP2/run_generation.py:62-134)."""

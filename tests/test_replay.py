@@ -54,6 +54,15 @@ def _rounding_reference(folder, requests):
         ops.set_backend(old)
 
 
+def _poisoned(runner):
+    """Every slot of the cache that no live request owns holds NaN: at the start all of them, later (the
+    runner's ``poison_freed_pages``) every page that is given back. A kernel that reads a slot beyond a
+    request's tokens, or a page that the request no longer owns, turns its logits into NaN."""
+    for kv in runner.kv_tensors:
+        kv.fill_(float("nan"))
+    return runner
+
+
 def _run_all_modes(make_runner, folder, dtype, rounding_reference=False):
     cfg, _ = plain.read_model_folder(folder)
     requests = _requests(cfg["vocab_size"])
@@ -87,7 +96,8 @@ def test_replay_on_emulated_kernels(model_folders, emulated_kernels, name, tmp_p
     from nanohybrid_vlm_amd.engine.runner import ModelRunner
 
     def make(folder, dtype, page, pages):
-        return ModelRunner(folder, dtype=dtype, device="cpu", page_size=page, num_pages=pages, num_state_slots=4)
+        return _poisoned(ModelRunner(folder, dtype=dtype, device="cpu", page_size=page, num_pages=pages,
+                                     num_state_slots=4, poison_freed_pages=True))
 
     folder = model_folders[name]
     if name != "C":
@@ -105,8 +115,8 @@ def test_replay_on_gpu(model_folders, name, dtype, graphs, tmp_path):
     from nanohybrid_vlm_amd.engine.runner import ModelRunner
 
     def make(folder, dtype, page, pages):
-        return ModelRunner(folder, dtype=dtype, device="cuda:0", page_size=page, num_pages=pages, num_state_slots=4,
-                           use_graphs=graphs, max_model_len=160)
+        return _poisoned(ModelRunner(folder, dtype=dtype, device="cuda:0", page_size=page, num_pages=pages,
+                                     num_state_slots=4, use_graphs=graphs, max_model_len=160, poison_freed_pages=True))
 
     folder = model_folders[name.split("_")[0]]
     if name.endswith("_sharp"):
@@ -158,8 +168,8 @@ def test_replay_at_the_family_head_size(model_folders, dtype, graphs):
         for mode, steps in [("whole", rc.whole(requests)), ("tail", rc.tail_decoded(requests, tail=40)),
                             ("mixed", rc.mixed(requests, sizes=(100, 7, 64, 2, 129, 33)))]:
             pages = rc.peak_tokens(steps, page) // page
-            runner = ModelRunner(folder, dtype=dtype, page_size=page, num_pages=pages, num_state_slots=4,
-                                 use_graphs=graphs, max_model_len=768)
+            runner = _poisoned(ModelRunner(folder, dtype=dtype, page_size=page, num_pages=pages, num_state_slots=4,
+                                           use_graphs=graphs, max_model_len=768, poison_freed_pages=True))
             got = rc.run_in_process(runner, steps)
             _check(got, want, tolerance_for(dtype, want), f"{dtype} head size 128, pages of {page}, {mode}")
 

@@ -24,8 +24,8 @@ class Clock:
 
 
 def make(pages=64, page=4, max_seqs=8, budget=16, policy="decode_first", wait_ms=50.0, slots=None, clock=None,
-         max_model_len=4096):
-    cache = CacheManager([PagedGroupSpec("all", page, pages)], slots or max_seqs)
+         max_model_len=4096, share_prefixes=False):
+    cache = CacheManager([PagedGroupSpec("all", page, pages)], slots or max_seqs, share_prefixes=share_prefixes)
     return Scheduler(cache, max_seqs, budget, EOS, max_model_len, policy, wait_ms, clock or Clock())
 
 
@@ -48,7 +48,8 @@ def run(s, prompts, params, next_fn=next_token, max_steps=10000, on_step=None, l
         for q in plan.seqs:
             n = q.num_scheduled_tokens
             assert n >= 1
-            s.cache.commit(q.seq_id, q.num_cached_tokens + n)          # what the runner does after the pass
+            # what the runner does after the pass
+            s.cache.commit(q.seq_id, q.num_cached_tokens + n, q.token_ids[q.num_cached_tokens:q.num_cached_tokens + n])
             ends = q.num_cached_tokens + n == q.num_tokens
             tokens.append(next_fn(q.token_ids) if ends else None)
         log.append({"decode": [q.seq_id for q in plan.decode_seqs],
@@ -209,3 +210,26 @@ def test_random_workloads_give_the_same_completions(seed):
              policy=rng.choice(["decode_first", "prefill_first"]))
     done, _ = run(s, prompts, params)
     assert done == {i: expected(p, sp.max_tokens) for i, (p, sp) in enumerate(zip(prompts, params))}
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_shared_prefixes_change_no_completion(seed):
+    """Prompts that start alike share pages; requests that are pushed out find their own pages again. The
+    completions are those of a run without sharing, and fewer tokens are computed."""
+    import random
+    rng = random.Random(100 + seed)
+    starts = [[rng.randrange(1, VOCAB) for _ in range(rng.randint(4, 20))] for _ in range(3)]
+    prompts = [rng.choice(starts) + [rng.randrange(1, VOCAB) for _ in range(rng.randint(0, 9))] for _ in range(12)]
+    params = [greedy(rng.randint(1, 12)) for _ in prompts]
+    pages = max(-(-(len(p) + sp.max_tokens) // 4) for p, sp in zip(prompts, params)) + rng.randint(0, 6)
+    options = dict(pages=pages, page=4, max_seqs=rng.randint(1, 5), budget=rng.randint(2, 20),
+                   policy=rng.choice(["decode_first", "prefill_first"]))
+    computed = {}
+    for share in (False, True):
+        s = make(share_prefixes=share, **options)
+        done, log = run(s, prompts, params)
+        assert done == {i: expected(p, sp.max_tokens) for i, (p, sp) in enumerate(zip(prompts, params))}
+        computed[share] = sum(len(e["decode"]) + sum(n for _, n in e["prefill"]) for e in log)
+        if share:
+            assert s.cache.num_shared_tokens > 0
+    assert computed[True] < computed[False]

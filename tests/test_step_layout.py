@@ -1,0 +1,86 @@
+"""The arrays that a step hands to the kernels: positions, slots, block tables, wanted rows and graph padding.
+Checked position by position with plain loops (the reference builds the same arrays in
+nanovllm/engine/model_runner.py:1406-1455 for prompts and :1516-1540 for single tokens)."""
+import random
+
+import numpy as np
+import pytest
+
+from nanohybrid_vlm_amd.cache.manager import OutOfPages
+from nanohybrid_vlm_amd.engine.runner import ModelRunner, StepEntry
+
+
+@pytest.fixture()
+def runner(model_folders, emulated_kernels):
+    return ModelRunner(model_folders["A"], dtype="float32", device="cpu", page_size=4, num_pages=40, num_state_slots=4)
+
+
+def _unpack(arrays):
+    input_ids, positions, token_req, cu, context_lens, state_slots, slot_mapping, bt = arrays
+    return dict(input_ids=input_ids, positions=positions, token_req=token_req, cu=cu, context_lens=context_lens,
+                state_slots=state_slots, slot_mapping=slot_mapping, bt=bt)
+
+
+def test_every_token_lands_on_its_slot(runner):
+    rng = random.Random(5)
+    lengths = {"a": 0, "b": 0, "c": 0}
+    tokens_of = {rid: [] for rid in lengths}
+    slot_of_position = {rid: {} for rid in lengths}
+    for step in range(12):
+        live = rng.sample(sorted(lengths), rng.randint(1, 3))
+        entries = []
+        for rid in live:
+            n = rng.choice([1, 1, 2, 3, 5, 9])
+            toks = [rng.randrange(runner.vocab_size) for _ in range(n)]
+            entries.append(StepEntry(rid, toks, [n - 1]))
+        arrays, meta = runner._layout(entries)
+        a = _unpack(arrays)
+        row = 0
+        for i, e in enumerate(entries):
+            table = runner.cache.block_table(e.request_id)
+            assert a["cu"][i] == row
+            assert a["context_lens"][i] == lengths[e.request_id] + len(e.tokens)
+            assert list(a["bt"][i, :len(table)]) == table and (a["bt"][i, len(table):] == -1).all()
+            for j, tok in enumerate(e.tokens):
+                p = lengths[e.request_id] + j
+                assert a["input_ids"][row] == tok
+                assert a["positions"][row] == p
+                assert a["token_req"][row] == i
+                assert a["slot_mapping"][row] == table[p // 4] * 4 + p % 4
+                slot_of_position[e.request_id][p] = int(a["slot_mapping"][row])
+                row += 1
+            assert meta["rows"][i] == row - 1
+            lengths[e.request_id] += len(e.tokens)
+            tokens_of[e.request_id] += e.tokens
+            runner.cache.commit(e.request_id, lengths[e.request_id])
+        assert a["cu"][len(entries)] == row == meta["T"]
+    # no slot is used by two positions, of one request or of two
+    all_slots = [s for m in slot_of_position.values() for s in m.values()]
+    assert len(set(all_slots)) == len(all_slots)
+
+
+def test_padding_rows_store_nothing(runner):
+    runner._layout([StepEntry("a", [1, 2, 3, 4, 5], [])])
+    runner.cache.commit("a", 5)
+    arrays, meta = runner._layout([StepEntry("a", [7], [0])], pad_to=4, table_width=6)
+    a = _unpack(arrays)
+    assert meta["B"] == 4 and meta["T"] == 4 and meta["rows"] == [0]
+    assert a["bt"].shape == (4, 6)
+    assert list(a["slot_mapping"][1:]) == [-1, -1, -1]              # nothing is stored for the padding
+    assert list(a["context_lens"][1:]) == [1, 1, 1] and (a["bt"][1:, 0] == 0).all()   # and they read a place that exists
+    assert a["positions"][0] == 5 and a["slot_mapping"][0] == runner.cache.block_table("a")[1] * 4 + 1
+
+
+def test_bad_entries_are_refused(runner):
+    with pytest.raises(ValueError, match="twice"):
+        runner._layout([StepEntry("a", [1], []), StepEntry("a", [2], [])])
+    with pytest.raises(ValueError, match="at least one token"):
+        runner._layout([StepEntry("a", [], [])])
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        runner._layout([StepEntry("a", [runner.vocab_size], [])])
+    with pytest.raises(ValueError, match="wanted place"):
+        runner._layout([StepEntry("b", [1, 2], [2])])
+    with pytest.raises(OutOfPages):
+        runner._layout([StepEntry("c", [1] * 161, [])])
+    runner.cache.check()
+    assert np.asarray(runner.cache.block_table("c")).size == 0     # all or nothing
