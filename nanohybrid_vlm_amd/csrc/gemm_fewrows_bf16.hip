@@ -1,0 +1,174 @@
+// y[M, N] = x[M, K] . w[N, K]^T (+ bias), or silu(x . wg^T) * (x . wu^T), in bfloat16 for up to 16
+// rows of x: the matrix products of a decoding step, whose time is the time to stream w from memory once.
+//
+// A block owns NT tiles of 16 rows of w (with GLU also their partners in the second matrix) and all
+// of K; its waves take equal, contiguous shares of K, whole cache lines each, and a wave's lanes load
+// 16 bytes each straight into the MFMA operand layout (v_mfma_f32_16x16x32_bf16: the w tile as the
+// 16 x 32 operand, the rows of x as the 32 x 16 one), several loads in flight before the first is used.
+// The waves' sums meet in LDS and are added in the order of the waves, so the result does not depend
+// on timing. Rows of x beyond M and columns beyond K read as zero.
+//
+// How many tiles a block takes, how many waves share K and how many loads a wave keeps in flight is
+// chosen per call from M, N and K (plan() below): blocks that spread evenly over the compute units
+// matter most, two tiles per block halve the reads of x when it has more than a few rows. (Splitting
+// K over several blocks, with the last one to arrive adding the parts in order, was measured and never
+// won: the fences cost more than the balance gains.)
+#include "nhv_common.h"
+
+namespace fewrows {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+// NT: tiles of 16 rows of w per block; WAVES: waves that share the block's part of K; UNROLL: loads in
+// flight per wave and operand. A step is 32 columns of K (64 bytes of a row).
+template <int NT, int WAVES, int UNROLL, bool GLU, typename TOut>
+__global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                  const bf16_t* __restrict__ bias, TOut* __restrict__ y,
+                                                                  int M, int N, int K, int steps_per_wave) {
+  constexpr int NA = GLU ? 2 : 1;
+  constexpr int TILES = NA * NT;
+  static_assert(NT <= WAVES, "wave nt finishes tile nt");
+  __shared__ float red[WAVES][TILES][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int n0 = blockIdx.x * 16 * NT;
+
+  const bf16_t* wrow[TILES];
+  bool n_ok[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = n0 + nt * 16 + col;
+    n_ok[nt] = n < N;
+#pragma unroll
+    for (int na = 0; na < NA; ++na) wrow[na * NT + nt] = w + ((size_t)na * N + (n_ok[nt] ? n : 0)) * K;
+  }
+  const bool m_ok = col < M;
+  const bf16_t* xrow = x + (size_t)(m_ok ? col : 0) * K;
+
+  floatx4 acc[TILES];
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int ksteps = (K + 31) / 32;
+  const int first = wave * steps_per_wave;
+  const int last = min(first + steps_per_wave, ksteps);
+  for (int s0 = first; s0 < last; s0 += UNROLL) {
+    bf16x8 a[UNROLL][TILES], b[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int k = (s0 + u) * 32 + grp * 8;
+      const bool k_ok = (s0 + u < last) && k < K;      // K is a multiple of 8: a piece is inside or outside as a whole
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) a[u][t] = (n_ok[t % NT] && k_ok) ? load8(wrow[t] + k) : zero8();
+      b[u] = (m_ok && k_ok) ? load8(xrow + k) : zero8();
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][t], b[u], acc[t], 0, 0, 0);
+  }
+#pragma unroll
+  for (int t = 0; t < TILES; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) red[wave][t][j][lane] = acc[t][j];
+  __syncthreads();
+  if (wave >= NT) return;
+
+  // wave nt adds the waves' sums of tile nt (and of its partner) in the order of the waves
+  const int nt = wave;
+  float v[NA][4];
+#pragma unroll
+  for (int na = 0; na < NA; ++na)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float sum = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) sum += red[wv][na * NT + nt][j][lane];
+      v[na][j] = sum;
+    }
+
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + nt * 16 + grp * 4 + j;           // the tile's row 4 grp + j is output n, its column is row col of x
+    if (col < M && n < N) {
+      float r = v[0][j];
+      if (bias) r += (float)bias[n];
+      if (GLU) r = r / (1.0f + expf(-r)) * v[NA - 1][j];
+      y[(size_t)col * N + n] = (TOut)r;
+    }
+  }
+}
+
+struct Plan {
+  int nt, waves, unroll;
+};
+
+// Chosen from measurements on an MI355X at the layer and head shapes of the 8B, 14B and 32B models
+// (N from 4096 to 151936, K from 4096 to 25600, M = 1, 2, 4, 8, 12, 16). The time of a variant followed
+//     (1 + M / (16 NT)) * penalty(NT) / evenness(blocks)
+// closely: the rows of x are read once per block, so their share falls with NT; two tiles per block cost
+// about an eighth for the parallelism they give up; and `evenness` is how full the last of the rounds of
+// 256 blocks (one per compute unit) is. Waves and loads in flight were then taken from the best variants.
+static Plan plan(bool glu, int M, int N, int K) {
+  const int tiles = (N + 15) / 16;
+  auto cost = [&](int nt) {
+    const int blocks = (tiles + nt - 1) / nt;
+    const int rounds = (blocks + 255) / 256;
+    const double evenness = (double)blocks / (256.0 * rounds);
+    return (1.0 + M / (16.0 * nt)) * (nt == 2 ? 1.13 : 1.0) / evenness;
+  };
+  const int nt = cost(2) < cost(1) ? 2 : 1;
+  if (glu) {
+    if (nt == 2) return {2, 8, 4};
+    return tiles <= 1024 ? Plan{1, 4, 8} : Plan{1, 8, 4};
+  }
+  if (nt == 2) return M <= 8 ? Plan{2, 8, 2} : Plan{2, 4, 4};
+  if (tiles > 256 && tiles < 512) return M <= 2 ? Plan{1, 4, 8} : Plan{1, 4, 4};
+  return {1, 8, 8};
+}
+
+template <int NT, int WAVES, int UNROLL, bool GLU>
+static void launch(hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
+                   int out_dtype) {
+  const int ksteps = (K + 31) / 32;
+  const int steps_per_wave = 2 * ((ksteps + 2 * WAVES - 1) / (2 * WAVES));     // even: whole cache lines of 128 bytes
+  const unsigned blocks = (unsigned)((N + 16 * NT - 1) / (16 * NT));
+  if (out_dtype == NHV_BF16)
+    hipLaunchKernelGGL((gemm_fewrows_kernel<NT, WAVES, UNROLL, GLU, bf16_t>), dim3(blocks), dim3(64 * WAVES), 0, s,
+                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, M, N, K, steps_per_wave);
+  else
+    hipLaunchKernelGGL((gemm_fewrows_kernel<NT, WAVES, UNROLL, GLU, float>), dim3(blocks), dim3(64 * WAVES), 0, s,
+                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (float*)y, M, N, K, steps_per_wave);
+}
+
+}  // namespace fewrows
+
+// The caller has checked sizes, alignment and types (1 <= M <= 16, K a multiple of 8).
+void nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
+                             int out_dtype, hipStream_t s) {
+  using namespace fewrows;
+  const Plan p = plan(glu, M, N, K);
+#define NHV_FEWROWS_CASE(NT_, WV_, UN_, GLU_)                                              \
+  if (p.nt == NT_ && p.waves == WV_ && p.unroll == UN_ && glu == GLU_) {                   \
+    launch<NT_, WV_, UN_, GLU_>(s, x, w, bias, y, M, N, K, out_dtype);                     \
+    return;                                                                                \
+  }
+  NHV_FEWROWS_CASE(1, 8, 8, false)
+  NHV_FEWROWS_CASE(1, 4, 8, false)
+  NHV_FEWROWS_CASE(1, 4, 4, false)
+  NHV_FEWROWS_CASE(2, 8, 2, false)
+  NHV_FEWROWS_CASE(2, 4, 4, false)
+  NHV_FEWROWS_CASE(1, 4, 8, true)
+  NHV_FEWROWS_CASE(1, 8, 4, true)
+  NHV_FEWROWS_CASE(2, 8, 4, true)
+#undef NHV_FEWROWS_CASE
+}

@@ -1,19 +1,13 @@
-// y[M, N] = x[M, K] . w[N, K]^T (+ bias) in bfloat16 for few rows (M <= 64): the
-// matrix product of a decoding step, where every weight is read once and the
-// time is the time to stream w from memory.
-//
-// A block owns 16 rows of w (16 outputs n) and all M rows of x. Its waves (2 to 16,
-// more of them where the grid alone would not fill the chip) split K
-// between them in interleaved runs of a few hundred bytes per row, so that together they read each row of w
-// front to back and every cache line is asked for by one wave only; a wave's lanes load 16 bytes each straight into the MFMA operand
-// layout (v_mfma_f32_16x16x32_bf16: w tile as the 16 x 32 operand, x rows as the
-// 32 x 16 one), with several loads in flight before the first is used. The waves'
-// partial sums meet in LDS and are added in the order of the waves, so the result
-// does not depend on timing. Rows of x beyond M and columns beyond K read as zero.
+// y[M, N] = x[M, K] . w[N, K]^T (+ bias) in bfloat16 for few rows (M <= 64): the entry points of the
+// matrix products of a decoding step, and the kernel for 17 to 64 rows. Up to 16 rows go to the kernel in
+// gemm_fewrows_bf16.hip.
 #include "nhv_common.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+void nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
+                             int out_dtype, hipStream_t s);
 
 __device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x8 sk_zero8() {
@@ -21,108 +15,6 @@ __device__ __forceinline__ bf16x8 sk_zero8() {
 #pragma unroll
   for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
   return z;
-}
-
-// MT: tiles of 16 rows of x; WAVES: waves that split K; UNROLL: loads in flight per wave and operand.
-// GLU: w holds two matrices of N rows each, gate above up; the block works on 16 rows of both with the same
-// rows of x and writes silu(gate) * up, so the packed projection's [M, 2N] result never exists in memory.
-template <int MT, int WAVES, int UNROLL, bool GLU, typename TOut>
-__global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                                 const bf16_t* __restrict__ bias, TOut* __restrict__ y,
-                                                                 int M, int N, int K) {
-  constexpr int NA = GLU ? 2 : 1;
-  __shared__ float red[WAVES][NA][MT][4][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int col = lane & 15, grp = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int n_a = n0 + col;                          // the row of w that this lane loads
-  const bool n_ok = n_a < N;
-  const bf16_t* wrow = w + (size_t)(n_ok ? n_a : 0) * K;
-  const bf16_t* wrow2 = wrow + (size_t)N * K;          // GLU: the matching row of the second matrix
-  const bf16_t* xrow[MT];
-  bool m_ok[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + col;
-    m_ok[mt] = m < M;
-    xrow[mt] = x + (size_t)(m_ok[mt] ? m : 0) * K;
-  }
-  floatx4 acc[NA][MT];
-#pragma unroll
-  for (int na = 0; na < NA; ++na)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[na][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  // a wave takes UNROLL consecutive steps of 32 at a time (UNROLL * 64 bytes of every row, whole cache lines),
-  // the waves of the block take such runs in turn
-  const int ksteps = (K + 31) / 32;
-  for (int run = wave; run * UNROLL < ksteps; run += WAVES) {
-    bf16x8 a[UNROLL], a2[UNROLL], b[UNROLL][MT];
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int k = (run * UNROLL + u) * 32 + grp * 8;
-      const bool k_ok = k < K;                       // K is a multiple of 8: a piece is inside or outside as a whole
-      a[u] = (n_ok && k_ok) ? sk_load8(wrow + k) : sk_zero8();
-      if (GLU) a2[u] = (n_ok && k_ok) ? sk_load8(wrow2 + k) : sk_zero8();
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) b[u][mt] = (m_ok[mt] && k_ok) ? sk_load8(xrow[mt] + k) : sk_zero8();
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        acc[0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][mt], acc[0][mt], 0, 0, 0);
-        if (GLU) acc[NA - 1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[u], b[u][mt], acc[NA - 1][mt], 0, 0, 0);
-      }
-  }
-#pragma unroll
-  for (int na = 0; na < NA; ++na)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) red[wave][na][mt][j][lane] = acc[na][mt][j];
-  __syncthreads();
-  // the waves share the tiles of the result between them; each sums the partial results in the order of the waves
-  for (int mt = wave; mt < MT; mt += WAVES) {
-    const int m = mt * 16 + col;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float v = 0.f, v2 = 0.f;
-#pragma unroll
-      for (int wv = 0; wv < WAVES; ++wv) {
-        v += red[wv][0][mt][j][lane];
-        if (GLU) v2 += red[wv][NA - 1][mt][j][lane];
-      }
-      const int n = n0 + grp * 4 + j;               // the tile's row 4 grp + j is output n, its column is row m of x
-      if (m < M && n < N) {
-        if (bias) v += (float)bias[n];
-        if (GLU) v = v / (1.0f + expf(-v)) * v2;
-        y[(size_t)m * N + n] = (TOut)v;
-      }
-    }
-  }
-}
-
-template <int MT, int WAVES, int UNROLL, bool GLU>
-static void sk_launch(unsigned blocks, hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M, int N,
-                      int K, int out_dtype) {
-  if (out_dtype == NHV_BF16)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, UNROLL, GLU, bf16_t>), dim3(blocks), dim3(64 * WAVES), 0, s,
-                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, M, N, K);
-  else
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, UNROLL, GLU, float>), dim3(blocks), dim3(64 * WAVES), 0, s,
-                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (float*)y, M, N, K);
-}
-
-template <int MT, int UNROLL, bool GLU>
-static void sk_by_waves(int waves, unsigned blocks, hipStream_t s, const void* x, const void* w, const void* bias, void* y,
-                        int M, int N, int K, int out_dtype) {
-  constexpr int TILES = (GLU ? 2 : 1) * MT;
-  constexpr int MAXW = TILES <= 2 ? 16 : TILES <= 4 ? 8 : 4;      // keeps the block's LDS at 32 KB
-  if (waves >= 16 && MAXW >= 16) sk_launch<MT, (MAXW >= 16 ? 16 : MAXW), UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else if (waves >= 8 && MAXW >= 8) sk_launch<MT, (MAXW >= 8 ? 8 : MAXW), UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else if (waves >= 4) sk_launch<MT, 4, UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else sk_launch<MT, 2, UNROLL, GLU>(blocks, s, x, w, bias, y, M, N, K, out_dtype);
 }
 
 // For 17 to 64 rows of x the rows of x are the larger share of what a wave loads, so here a wave keeps NT
@@ -257,33 +149,17 @@ static int sk_check(const char* what, const void* x, const void* w, int M, int N
   return 0;
 }
 
-// enough waves in flight to cover the memory's latency: about 16 per compute unit over the whole grid,
-// but no wave with less than one round of loads
-static int sk_waves(unsigned blocks, int K) {
-  const int ksteps = (K + 31) / 32;
-  int waves = 2;
-  while (waves < 16 && (long long)blocks * waves < 4096 && ksteps >= waves * 2 * 4) waves *= 2;
-  return waves;
-}
-
 extern "C" int nhv_gemm_skinny_bf16(const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
                                     int out_dtype, void* stream) {
   if (sk_check("skinny gemm", x, w, M, N, K, out_dtype)) return 1;
-  const unsigned blocks = (unsigned)((N + 15) / 16);
   hipStream_t s = (hipStream_t)stream;
-  const int mt = (M + 15) / 16;
-  if (mt >= 2) {
+  if (M > 16) {
     mid_dispatch<false>(s, x, w, bias, y, M, N, K, out_dtype);
     NHV_LAUNCH_CHECK("gemm_mid_bf16");
     return 0;
   }
-  const int waves = sk_waves(blocks, K);
-  // long runs per wave (1 KB of every row in flight) where K is long enough to give every wave two of them
-  if (mt == 1 && (K + 31) / 32 >= waves * 32) sk_by_waves<1, 16, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else if (mt == 1) sk_by_waves<1, 8, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else if (mt == 2) sk_by_waves<2, 8, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  else sk_by_waves<4, 4, false>(waves, blocks, s, x, w, bias, y, M, N, K, out_dtype);
-  NHV_LAUNCH_CHECK("gemm_skinny_bf16");
+  nhv_gemm_fewrows_launch(false, x, w, bias, y, M, N, K, out_dtype, s);
+  NHV_LAUNCH_CHECK("gemm_fewrows_bf16");
   return 0;
 }
 
@@ -291,18 +167,13 @@ extern "C" int nhv_gemm_skinny_bf16(const void* x, const void* w, const void* bi
 extern "C" int nhv_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_dtype,
                                         void* stream) {
   if (sk_check("skinny gated gemm", x, w, M, N, K, out_dtype)) return 1;
-  const unsigned blocks = (unsigned)((N + 15) / 16);
   hipStream_t s = (hipStream_t)stream;
-  const int mt = (M + 15) / 16;
-  if (mt >= 2) {
+  if (M > 16) {
     mid_dispatch<true>(s, x, w, nullptr, y, M, N, K, out_dtype);
     NHV_LAUNCH_CHECK("gemm_mid_glu_bf16");
     return 0;
   }
-  const int waves = sk_waves(blocks, K);
-  if (mt == 1) sk_by_waves<1, 8, true>(waves, blocks, s, x, w, nullptr, y, M, N, K, out_dtype);
-  else if (mt == 2) sk_by_waves<2, 4, true>(waves, blocks, s, x, w, nullptr, y, M, N, K, out_dtype);
-  else sk_by_waves<4, 4, true>(waves, blocks, s, x, w, nullptr, y, M, N, K, out_dtype);
-  NHV_LAUNCH_CHECK("gemm_skinny_glu_bf16");
+  nhv_gemm_fewrows_launch(true, x, w, nullptr, y, M, N, K, out_dtype, s);
+  NHV_LAUNCH_CHECK("gemm_fewrows_glu_bf16");
   return 0;
 }

@@ -134,7 +134,24 @@ def test_skinny_linear_bfloat16(ops, M, N, K):
                                    ops.linear(x, w, out_dtype=torch.float32)[:1], rtol=1e-5, atol=1e-5)
 
 
-@pytest.mark.parametrize("M,I,K", [(1, 112, 80), (5, 1001, 96), (16, 12288, 4096), (17, 160, 96), (64, 300, 1024)])
+@pytest.mark.parametrize("M,N,K", [
+    # every way the kernel for up to 16 rows cuts the work: one or two tiles of 16 outputs per block, 4 or 8 waves
+    (1, 6144, 264), (2, 5000, 4096), (5, 7168, 72), (8, 6100, 1032), (12, 5120, 520), (16, 151936, 64), (9, 10240, 40),
+    (16, 16, 8), (3, 17, 25608),
+])
+def test_few_rows_linear_bfloat16_in_all_its_variants(ops, M, N, K):
+    x = rnd(M, K, dtype=torch.bfloat16, seed=34)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=35, scale=K ** -0.5)
+    b = rnd(N, dtype=torch.bfloat16, seed=36)
+    ref = x.double() @ w.double().T
+    torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32).double(), ref, rtol=1e-4, atol=2e-4)
+    torch.testing.assert_close(ops.linear(x, w, b).double(), ref + b.double(), **tol(torch.bfloat16))
+    # the same call twice gives the same bits: the sums are added in a fixed order
+    assert torch.equal(ops.linear(x, w, out_dtype=torch.float32), ops.linear(x, w, out_dtype=torch.float32))
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 112, 80), (5, 1001, 96), (16, 12288, 4096), (17, 160, 96), (64, 300, 1024),
+                                   (4, 17408, 136), (16, 25600, 72), (13, 25000, 264)])
 def test_gated_linear(ops, M, I, K):
     """silu(x Wg^T) * (x Wu^T): the fused kernel for few rows, the two-kernel way for many; float32 as well."""
     for dtype in DTYPES:
