@@ -15,12 +15,20 @@
 // order of the slots is free as long as P and V agree), so P never goes through
 // memory, and because the second product is taken transposed a lane's output entries
 // belong to the same row as its scores: the rescaling needs no exchange between lanes.
-// V is written to LDS transposed, four keys (8 bytes) at a time; the columns of that
-// tile are XOR-ed with the row's 8-group so that a wave's writes fall into distinct banks.
-// The next tile's keys and values are asked for from memory before the current tile
-// is computed. A query at position p reads keys lo..p (lo = p - window + 1 with a
-// window, else 0). Keys outside the block's range are staged as zeros: unused cache
-// slots may hold anything, and 0 * NaN would poison the sums.
+//
+// Keys and values go from the cache straight into LDS (global_load_lds, 16 bytes a lane,
+// no registers in between), row by row as they lie in the cache, into one of two
+// buffers: the next tile is on its way while this one is computed, and a tile costs one
+// barrier. Such a load puts lane i's piece at the wave's LDS base + 16 i, so the layout
+// is linear; bank conflicts are avoided by which piece of the row a lane asks for (the
+// piece index XOR-ed with the key's low bits). The V^T operand is read from the
+// row-major tile with ds_read_b64_tr_b16: in a group of 16 lanes, lane i receives
+// element i % 4 of the 8-byte pieces that lanes i / 4 + 4 j (j = 0..3) point at, so with
+// lane r pointing at key r / 4, entries 4 (r % 4).. of the 16-entry block, lane i gets
+// entry i of four consecutive keys. A query at position p reads keys lo..p (lo = p -
+// window + 1 with a window, else 0). Keys outside the block's range are replaced by the
+// nearest key inside it (their P is 0): unused cache slots may hold anything, and 0 * NaN
+// would poison the sums.
 #include "nhv_common.h"
 #include <math.h>
 
@@ -38,16 +46,21 @@ static_assert(D % 16 == 0 && D >= 16, "head size must be a multiple of 16");
 constexpr bool SUPPORTED = D <= 256;        // beyond that the tiles do not fit into 64 KB of LDS
 constexpr int BN = D <= 128 ? 64 : 32;      // keys per tile
 constexpr int KT = BN / 16;                 // 16-key sub-tiles
-constexpr int KPITCH = DSTEPS * 32 + 8;     // elements per row of the K tile (padded against bank conflicts)
-constexpr int VPITCH = BN + 8;              // elements per row of the transposed V tile
-constexpr int QUADS = (BN / 4) * CH;        // (4 keys, 16-byte piece) units of a tile
-constexpr int QPT = (QUADS + 255) / 256;    // of them per thread
-constexpr int SWZ_MASK = BN / 4 - 1;        // column of key k in row d of the V^T tile: k ^ (((d >> 3) & SWZ_MASK) << 2)
+constexpr int PIECES = BN * CH;             // 16-byte pieces of a tile of keys (or of values)
+constexpr int LOADS = (PIECES + 255) / 256; // direct loads per thread, tile and matrix
+constexpr bool CH_POW2 = (CH & (CH - 1)) == 0;
+// piece c of key k lies at piece c ^ (k & KSWZ) of its row in the K tile: 16 keys read the same piece at once
+constexpr int KSWZ = CH_POW2 ? (CH < 16 ? CH : 16) - 1 : 0;
+// and at c ^ ((k & VSWZ) << 1) in the V tile, whose transposed reads take 32 bytes of 8 keys at once
+constexpr int VSWZ = CH_POW2 && CH >= 4 ? (CH / 2 < 8 ? CH / 2 : 8) - 1 : 0;
 constexpr int TPB = 4;                      // row tiles per block, one per wave
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
+typedef const __attribute__((address_space(1))) void* global_ptr;
 
 __device__ __forceinline__ bf16x8 zero8() {
   bf16x8 z;
@@ -73,8 +86,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
     const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv, int page_size, int page_shift,
     float scale_log2e, int window) {
   constexpr int DL = SUPPORTED ? D : 16;                   // keeps the unsupported sizes compilable; they are never launched
-  __shared__ __attribute__((aligned(16))) bf16_t k_s[BN * (SUPPORTED ? KPITCH : 24)];
-  __shared__ __attribute__((aligned(16))) bf16_t vt_s[DL * VPITCH];
+  constexpr int TILE = SUPPORTED ? BN * DL : 16;           // elements of a tile
+  __shared__ __attribute__((aligned(16))) bf16_t k_s0[TILE], k_s1[TILE], v_s0[TILE], v_s1[TILE];
   __shared__ int bt_s[BT_IN_LDS ? BT_LDS : 1];
   if (!SUPPORTED) return;
 
@@ -142,75 +155,34 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
     return BT_IN_LDS ? slot_of((const int*)bt_s, key, page_size, page_shift) : slot_of(bt_g, key, page_size, page_shift);
   };
 
-  // staging: a thread owns the same 16-byte piece of four consecutive keys
-  bf16x8 kreg[QPT][4], vreg[QPT][4];
-  auto fetch = [&](int kb) {                               // memory -> registers
-    const bool whole = kb >= key_lo && kb + BN - 1 <= key_hi;    // every key of the tile is in range (all but the ends)
+  // memory -> LDS without registers: wave w's load number i brings pieces (4 i + w) * 64 + lane of the tile
+  auto issue = [&](int kb, bf16_t* k_s, bf16_t* v_s) {
 #pragma unroll
-    for (int i = 0; i < QPT; ++i) {
-      const int u = tid + i * 256;
-      const int kq = u / CH, dc = u % CH;
-      if (whole && (QUADS % 256 == 0 || u < QUADS)) {
-#pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) {
-          const size_t off = ((size_t)slot(kb + kq * 4 + k4) * Hkv + kvh) * D + dc * 8;
-          kreg[i][k4] = *reinterpret_cast<const bf16x8*>(k_cache + off);
-          vreg[i][k4] = *reinterpret_cast<const bf16x8*>(v_cache + off);
-        }
-        continue;
-      }
-#pragma unroll
-      for (int k4 = 0; k4 < 4; ++k4) {
-        const int key = kb + kq * 4 + k4;
-        kreg[i][k4] = zero8();
-        vreg[i][k4] = zero8();
-        if (u < QUADS && key >= key_lo && key <= key_hi) {
-          const size_t off = ((size_t)slot(key) * Hkv + kvh) * D + dc * 8;
-          kreg[i][k4] = *reinterpret_cast<const bf16x8*>(k_cache + off);
-          vreg[i][k4] = *reinterpret_cast<const bf16x8*>(v_cache + off);
-        }
-      }
-    }
-  };
-  auto stash = [&]() {                                     // registers -> LDS: K as it is, V transposed
-#pragma unroll
-    for (int i = 0; i < QPT; ++i) {
-      const int u = tid + i * 256;
-      if (u < QUADS) {
-        const int kq = u / CH, dc = u % CH;
-#pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) *reinterpret_cast<bf16x8*>(k_s + (kq * 4 + k4) * KPITCH + dc * 8) = kreg[i][k4];
-        const int vcol = (kq * 4) ^ ((dc & SWZ_MASK) << 2);  // (d >> 3) is dc for all eight entries of the piece
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          bf16x4 four;
-#pragma unroll
-          for (int k4 = 0; k4 < 4; ++k4) four[k4] = vreg[i][k4][e];
-          *reinterpret_cast<bf16x4*>(vt_s + (dc * 8 + e) * VPITCH + vcol) = four;
-        }
+    for (int i = 0; i < LOADS; ++i) {
+      const int u = (i * 4 + wave) * 64 + lane;
+      if (PIECES % 256 == 0 || u < PIECES) {
+        const int kl = u / CH, piece = u % CH;
+        const int key = min(max(kb + kl, key_lo), key_hi);
+        const size_t row = ((size_t)slot(key) * Hkv + kvh) * D;
+        const size_t koff = row + (piece ^ (kl & KSWZ)) * 8;
+        const size_t voff = row + (piece ^ ((kl & VSWZ) << 1)) * 8;
+        __builtin_amdgcn_global_load_lds((global_ptr)(k_cache + koff), (lds_ptr)(k_s + (i * 4 + wave) * 512), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((global_ptr)(v_cache + voff), (lds_ptr)(v_s + (i * 4 + wave) * 512), 16, 0, 0);
       }
     }
   };
 
-  if (D % 32 != 0) {                                       // the padded half step of the first product reads zeros
-    for (int c = tid; c < BN * 2; c += 256) *reinterpret_cast<bf16x8*>(k_s + (c / 2) * KPITCH + D + (c % 2) * 8) = zero8();
-  }
-  const int kb0 = (key_lo / BN) * BN;
-  fetch(kb0);
-  for (int kb = kb0; kb <= key_hi; kb += BN) {
-    __syncthreads();                                       // the last tile has been read by every wave
-    stash();
-    __syncthreads();
-    if (kb + BN <= key_hi) fetch(kb + BN);                 // in flight while this tile is computed
-    if (!live || kb > wave_hi) continue;                   // a whole-wave decision; the wave still meets the barriers
-    // ---- scores of 64 keys for this wave's 16 rows
+  auto compute = [&](int kb, const bf16_t* k_s, const bf16_t* v_s) {
+    // ---- scores of the tile's keys for this wave's 16 rows
     floatx4 s4[KT];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
       s4[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < DSTEPS; ++s) {
-        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(k_s + (kt * 16 + col) * KPITCH + s * 32 + grp * 8);
+        const int piece = s * 4 + grp;
+        const bf16x8 ka = piece < CH ? *reinterpret_cast<const bf16x8*>(k_s + (kt * 16 + col) * D + (piece ^ (col & KSWZ)) * 8)
+                                     : zero8();
         s4[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[s], s4[kt], 0, 0, 0);
       }
     }
@@ -249,28 +221,45 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
       }
     l_part = l_part * alpha + psum;
     m_run = m_new;
+    // this lane points at key 4 grp + col / 4 of a 16-key sub-tile, entries 4 (col % 4).. of the 16-entry block dt
+    const int tr_key = grp * 4 + (col >> 2);
+    const int tr_piece = (col & 3) >> 1, tr_half = (col & 1) * 4;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
-      const int drow = dt * 16 + col;                      // the V^T row this lane reads as operand
-      const int swz = ((drow >> 3) & SWZ_MASK) << 2;
       if (grow) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
       }
 #pragma unroll
       for (int a = 0; a < KT / 2; ++a) {
-        // this lane's eight summation slots: keys 32 a + 4 grp + (0..3) and 32 a + 16 + 4 grp + (0..3)
-        const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vt_s + drow * VPITCH + ((a * 32 + grp * 4) ^ swz));
-        const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vt_s + drow * VPITCH + ((a * 32 + 16 + grp * 4) ^ swz));
-        bf16x8 va;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          va[j] = lo4[j];
-          va[4 + j] = hi4[j];
-        }
+        // this lane's eight summation slots: keys 32 a + 4 grp + (0..3) and 32 a + 16 + 4 grp + (0..3), entry dt * 16 + col
+        const int k_lo = a * 32 + tr_key, k_hi = k_lo + 16;
+        const bf16_t* p_lo = v_s + k_lo * D + ((dt * 2 + tr_piece) ^ ((k_lo & VSWZ) << 1)) * 8 + tr_half;
+        const bf16_t* p_hi = v_s + k_hi * D + ((dt * 2 + tr_piece) ^ ((k_hi & VSWZ) << 1)) * 8 + tr_half;
+        const short4_t lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)p_lo);
+        const short4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)p_hi);
+        typedef short short8_t __attribute__((ext_vector_type(8)));
+        const short8_t both = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+        const bf16x8 va = __builtin_bit_cast(bf16x8, both);
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pa[a], o[dt], 0, 0, 0);
       }
     }
+  };
+
+  // tiles alternate between the two buffers; the loop is written out for both so that every load and read names
+  // its buffer (the compiler then knows that the loads under way do not touch the tile being read)
+  const int kb0 = (key_lo / BN) * BN;
+  issue(kb0, k_s0, v_s0);
+  for (int kb = kb0; kb <= key_hi; kb += 2 * BN) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();                                       // this tile has arrived, the other buffer has been read
+    if (kb + BN <= key_hi) issue(kb + BN, k_s1, v_s1);
+    if (live && kb <= wave_hi) compute(kb, k_s0, v_s0);    // a whole-wave decision; the wave still meets the barriers
+    if (kb + BN > key_hi) break;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (kb + 2 * BN <= key_hi) issue(kb + 2 * BN, k_s0, v_s0);
+    if (live && kb + BN <= wave_hi) compute(kb + BN, k_s1, v_s1);
   }
   if (!live) return;
   float l = l_part;
