@@ -55,3 +55,11 @@ def test_model_or_random_weights_is_needed():
     proc = subprocess.run([sys.executable, "-m", "nanohybrid_vlm_amd", "generate", "--prompt-ids", "1"], cwd=REPO,
                           capture_output=True, text=True, timeout=120)
     assert proc.returncode != 0 and "--model DIR or --random-weights SEED" in proc.stderr
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The measurement program is for one GPU: for more it says so in one line and exits with 2."""
+    proc = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), "--gpus", "2", "--steps", "1", "--warmup", "0"],
+                          cwd=REPO, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 2
+    assert len(proc.stdout.strip().splitlines()) == 1 and "one GPU" in proc.stdout
