@@ -16,6 +16,8 @@
 // key positions. Each split writes its unnormalised output with (maximum, sum) in
 // float; a second kernel merges the splits in rising order. Keys that are not visible
 // are loaded as zeros (the cache's unused slots may hold anything).
+// (Asking for the next round before this one is computed was measured: the second set of
+// registers leaves one wave per SIMD, and that costs more than the overlap gains.)
 #include "nhv_common.h"
 #include <math.h>
 
