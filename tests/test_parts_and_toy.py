@@ -1,8 +1,10 @@
 """The parts are general: a toy architecture, defined here and nowhere in the package,
-with a mixer that keeps state of its own per request, a layer with a window (pages of
-its own, given back as the window passes), a layer that runs twice and an entry that
-reads another entry's cache, is registered, built, loaded and stepped through the
-unchanged engine and compared with a plain whole-sequence computation.
+with a mixer that keeps state of its own per request, a feed-forward that routes every
+token to one of several experts, a position encoding of its own (other angles, on a
+part of the head only), a layer with a window (pages of its own, given back as the
+window passes), a layer that runs twice and an entry that reads another entry's cache,
+is registered, built, loaded and stepped through the unchanged engine and compared
+with a plain whole-sequence computation.
 Also: each built-in part alone against its plain function."""
 import pytest
 import torch
@@ -13,11 +15,12 @@ from helpers import max_abs_diff
 from nanohybrid_vlm_amd.cache.manager import NO_PAGE
 from nanohybrid_vlm_amd.config.registry import (Architecture, WeightSource, register_architecture,
                                                 unregister_architecture)
-from nanohybrid_vlm_amd.parts import MIXERS, ParamSpec, Part, StateNeed
+from nanohybrid_vlm_amd.parts import FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, ParamSpec, Part, StateNeed
 from nanohybrid_vlm_amd.parts.model import DecoderModel, LayerSpec, ModelSpec, RunEntry
 from nanohybrid_vlm_amd.weights.random_init import write_random_model
 
 H, HEADS, KV, D, INTER, VOCAB, WINDOW, DECAY = 48, 3, 1, 16, 64, 97, 5, 0.75
+EXPERTS, EXPERT_INTER, TOY_ROT, TOY_STEP = 3, 40, 8, 0.05
 
 
 class DecayingSum(Part):
@@ -50,6 +53,53 @@ class DecayingSum(Part):
         return out
 
 
+class RoutedFeedForward(Part):
+    """Toy feed-forward with routing: router logits and their softmax in float32; every token goes through
+    the expert it rates highest (the experts are the package's own gated feed-forwards, built through the
+    registry) and the result is weighted with that expert's probability."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int):
+        self.hidden_size = hidden_size
+        self.experts = [FEED_FORWARDS.build({"kind": "swiglu", "hidden_size": hidden_size,
+                                             "intermediate_size": intermediate_size}) for _ in range(num_experts)]
+
+    def param_specs(self):
+        return {"router.weight": ParamSpec((len(self.experts), self.hidden_size), keeps_float32=True)}
+
+    def children(self):
+        return {f"experts.{i}": e for i, e in enumerate(self.experts)}
+
+    def bind(self, params):
+        self.router = params["router.weight"]
+
+    def forward(self, x, step):
+        prob = torch.softmax(x.float() @ self.router.float().T, dim=-1)
+        best = prob.argmax(dim=-1)
+        out = torch.zeros_like(x)
+        for e, expert in enumerate(self.experts):
+            rows = (best == e).nonzero().flatten()
+            if rows.numel():
+                y = expert.forward(x[rows].contiguous(), step)
+                out[rows] = (y.float() * prob[rows, e:e + 1]).to(x.dtype)
+        return out
+
+
+class LinearAngles(Part):
+    """Toy position encoding: the angle of pair j at position p is p * (j + 1) * step, and only the first
+    ``rotary_dim`` entries of a head are turned."""
+
+    def __init__(self, rotary_dim: int, step: float, max_position: int, device=None):
+        ang = torch.arange(max_position, dtype=torch.float32)[:, None] * (torch.arange(rotary_dim // 2) + 1.0) * step
+        self.table = torch.cat((ang.cos(), ang.sin()), dim=-1).contiguous()
+
+    def rotation_table(self):
+        return self.table
+
+    def to(self, device):
+        self.table = self.table.to(device)
+        return self
+
+
 def toy_spec(cfg: dict) -> ModelSpec:
     norm = {"kind": "rmsnorm", "size": H, "eps": 1e-5}
     ff = {"kind": "swiglu", "hidden_size": H, "intermediate_size": INTER}
@@ -57,15 +107,17 @@ def toy_spec(cfg: dict) -> ModelSpec:
     def attention(window):
         return {"kind": "gqa_attention", "hidden_size": H, "num_heads": HEADS, "num_kv_heads": KV, "head_dim": D,
                 "scale": D ** -0.5, "qk_norm_eps": 1e-5, "qkv_bias": False, "window": window}
+    routed = {"kind": "toy_routed", "hidden_size": H, "intermediate_size": EXPERT_INTER, "num_experts": EXPERTS}
     layers = [
         LayerSpec(mixer=attention(None), feed_forward=ff, norm=norm),
-        LayerSpec(mixer={"kind": "toy_decaying_sum", "hidden_size": H, "decay": DECAY}, feed_forward=ff, norm=norm),
-        LayerSpec(mixer=attention(WINDOW), feed_forward=ff, norm=norm),
+        LayerSpec(mixer={"kind": "toy_decaying_sum", "hidden_size": H, "decay": DECAY}, feed_forward=routed, norm=norm),
+        LayerSpec(mixer=attention(WINDOW), feed_forward=ff, norm=norm, position="linear"),
     ]
     # layer 0 runs twice (two caches); the last entry runs layer 2 again on the keys and values of entry 2
     order = [RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(2, cache=2)]
     return ModelSpec(vocab_size=VOCAB, hidden_size=H, layers=layers, final_norm=norm,
-                     positions={"default": {"kind": "rope", "rotary_dim": D, "base": 1000.0}},
+                     positions={"default": {"kind": "rope", "rotary_dim": D, "base": 1000.0},
+                                "linear": {"kind": "toy_linear_angles", "rotary_dim": TOY_ROT, "step": TOY_STEP}},
                      max_position=256, tie_embeddings=True, run_order=order)
 
 
@@ -75,11 +127,31 @@ def toy_names(cfg):
 
 @pytest.fixture()
 def toy_architecture():
-    MIXERS.register("toy_decaying_sum")(DecayingSum)
+    _register_toy_parts()
     register_architecture(Architecture("ToyForCausalLM", ("toy",), dict, toy_spec, toy_names))
     yield
     unregister_architecture("ToyForCausalLM")
+    _unregister_toy_parts()
+
+
+def _register_toy_parts():
+    MIXERS.register("toy_decaying_sum")(DecayingSum)
+    FEED_FORWARDS.register("toy_routed")(RoutedFeedForward)
+    POSITION_ENCODINGS.register("toy_linear_angles")(LinearAngles)
+
+
+def _unregister_toy_parts():
     MIXERS.unregister("toy_decaying_sum")
+    FEED_FORWARDS.unregister("toy_routed")
+    POSITION_ENCODINGS.unregister("toy_linear_angles")
+
+
+def toy_turn(x, pos):
+    """The toy position encoding on [T, heads, D]: pairs (j, j + TOY_ROT / 2) of the first TOY_ROT entries."""
+    ang = pos.float()[:, None] * (torch.arange(TOY_ROT // 2) + 1.0) * TOY_STEP
+    cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+    x1, x2 = x[..., :TOY_ROT // 2], x[..., TOY_ROT // 2:TOY_ROT]
+    return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., TOY_ROT:]), dim=-1)
 
 
 def toy_plain_logits(w, toks):
@@ -90,15 +162,26 @@ def toy_plain_logits(w, toks):
     kept = {}
 
     def attention(x, p, window, entry, lender=None):
+        turn = toy_turn if window else (lambda t, at: plain.apply_rope(t, at, 1000.0))   # the windowed layer has the toy angles
         qkv = x @ w[p + "mixer.qkv.weight"].T
         q = plain.rms_norm(qkv[:, :HEADS * D].view(T, HEADS, D), w[p + "mixer.q_norm.weight"], 1e-5)
         if lender is None:
             k = plain.rms_norm(qkv[:, HEADS * D:(HEADS + KV) * D].view(T, KV, D), w[p + "mixer.k_norm.weight"], 1e-5)
             v = qkv[:, (HEADS + KV) * D:].view(T, KV, D)
-            kept[entry] = (plain.apply_rope(k, pos, 1000.0), v)
+            kept[entry] = (turn(k, pos), v)
         k, v = kept[entry if lender is None else lender]
-        o = plain.causal_attention(plain.apply_rope(q, pos, 1000.0), k, v, D ** -0.5, window)
+        o = plain.causal_attention(turn(q, pos), k, v, D ** -0.5, window)
         return o.reshape(T, HEADS * D) @ w[p + "mixer.o.weight"].T
+
+    def routed(x, p):
+        prob = torch.softmax(x @ w[p + "feed_forward.router.weight"].T, dim=-1)
+        rows = []
+        for t in range(T):
+            e = int(prob[t].argmax())
+            gu = w[p + f"feed_forward.experts.{e}.gate_up.weight"]
+            y = plain.swiglu(x[t:t + 1], gu[:EXPERT_INTER], gu[EXPERT_INTER:], w[p + f"feed_forward.experts.{e}.down.weight"])
+            rows.append(y[0] * prob[t, e])
+        return torch.stack(rows)
 
     def decaying_sum(x, p):
         s, rows = torch.zeros(H), []
@@ -115,6 +198,9 @@ def toy_plain_logits(w, toks):
         else:
             r = r + attention(x, p, WINDOW if layer == 2 else None, entry, lender)
         x = plain.rms_norm(r, w[p + "feed_forward_norm.weight"], 1e-5)
+        if layer == 1:
+            r = r + routed(x, p)
+            continue
         gu = w[p + "feed_forward.gate_up.weight"]
         r = r + plain.swiglu(x, gu[:INTER], gu[INTER:], w[p + "feed_forward.down.weight"])
     return plain.rms_norm(r, w["final_norm.weight"], 1e-5) @ w["embed.weight"].T
@@ -158,7 +244,7 @@ def test_toy_architecture_on_gpu(toy_architecture, dtype, tol, tmp_path):
 
 def test_run_order_is_checked():
     spec = toy_spec({})
-    MIXERS.register("toy_decaying_sum")(DecayingSum)
+    _register_toy_parts()
     try:
         spec.run_order = [RunEntry(0), RunEntry(5)]
         with pytest.raises(ValueError, match="names layer 5"):
@@ -170,8 +256,8 @@ def test_run_order_is_checked():
         with pytest.raises(ValueError, match="earlier entry"):
             DecoderModel(spec)
     finally:
-        MIXERS.unregister("toy_decaying_sum")
-    with pytest.raises(KeyError, match="unknown mixer"):
+        _unregister_toy_parts()
+    with pytest.raises(KeyError, match="unknown position encoding"):
         DecoderModel(toy_spec({}))
 
 
