@@ -2,11 +2,14 @@
 // cache in bfloat16 on the matrix cores. Compiled for one head size:
 // -DNHV_HEAD_DIM=<multiple of 16>.
 //
-// A block of 4 waves works on one (request, key/value head) and four row tiles, one per
-// wave; a row tile is 16 consecutive tokens of one query head, and the row tiles of a
-// request are numbered so that the heads sharing the key/value head come first: with 4
-// heads per key/value head a block is 16 tokens x 4 heads, and every key and value it
-// stages in LDS is used by 64 rows. Keys are taken in tiles of 64, in rising order:
+// A block of 4 waves works on one (request, key/value head) and four or eight row tiles,
+// one or two per wave; a row tile is 16 consecutive tokens of one query head, and the row
+// tiles of a request are numbered so that the heads sharing the key/value head come
+// first: with 4 heads per key/value head a block is 16 or 32 tokens x 4 heads, and every
+// key and value it stages in LDS is used by 64 or 128 rows. With two row tiles a wave
+// reads every operand of keys and values from LDS once for both (the reads from LDS are
+// what the kernel waits for most); that is taken where the batch still fills the chip
+// with blocks of that size. Keys are taken in tiles of 64, in rising order:
 //   S^T[key, row] = K[key, :] . Q[row, :]      K tile from LDS, Q in registers (v_mfma_f32_16x16x32_bf16)
 //   running maximum per row in float (two shuffles over the lane groups), sums kept per lane
 //   O^T[d, row]  += V^T[d, key] . P^T[key, row]  V^T from LDS, P in registers (v_mfma_f32_16x16x32_bf16)
@@ -53,7 +56,8 @@ constexpr bool CH_POW2 = (CH & (CH - 1)) == 0;
 constexpr int KSWZ = CH_POW2 ? (CH < 16 ? CH : 16) - 1 : 0;
 // and at c ^ ((k & VSWZ) << 1) in the V tile, whose transposed reads take 32 bytes of 8 keys at once
 constexpr int VSWZ = CH_POW2 && CH >= 4 ? (CH / 2 < 8 ? CH / 2 : 8) - 1 : 0;
-constexpr int TPB = 4;                      // row tiles per block, one per wave
+constexpr int MAX_RT = D <= 128 ? 2 : 1;    // row tiles per wave (template argument RT): all of them use every key and value
+                                            // that the wave reads from LDS; two need the registers of head sizes up to 128
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
@@ -79,8 +83,8 @@ __device__ __forceinline__ int slot_of(P bt, int key, int page_size, int page_sh
 
 // BT_IN_LDS: the request's block table (up to the block's last key) is copied into LDS first, so that the
 // look-up that every load of a key depends on costs an LDS read instead of a trip to memory.
-template <bool BT_IN_LDS>
-__global__ __launch_bounds__(256) void prefill_attention_kernel(
+template <bool BT_IN_LDS, int RT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void prefill_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens_q, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv, int page_size, int page_shift,
@@ -90,6 +94,7 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t k_s0[TILE], k_s1[TILE], v_s0[TILE], v_s1[TILE];
   __shared__ int bt_s[BT_IN_LDS ? BT_LDS : 1];
   if (!SUPPORTED) return;
+  constexpr int TPB = 4 * RT;                              // row tiles per block
 
   const int req = blockIdx.z, kvh = blockIdx.y;
   const int G = Hq / Hkv;
@@ -118,31 +123,45 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
   const int key_hi = start_pos + blk_tok_hi;
   const int key_lo = window > 0 ? max(0, start_pos + blk_tok_lo - window + 1) : 0;
 
-  // this wave's row tile; this lane's row (in both products) is token tok0 + col of the tile's head
-  const int my_tile = first_tile + wave;
-  const bool live = my_tile < n_row_tiles;
-  const int head = kvh * G + (live ? my_tile % G : 0);
-  const int tok0 = live ? (my_tile / G) * 16 : 0;
-  const int row_tok = tok0 + col;
-  const bool row_ok = live && row_tok < q_len;
-  const int row_pos = start_pos + min(row_tok, q_len - 1);
-  const int row_lo = window > 0 ? max(0, row_pos - window + 1) : 0;
-  const int wave_lo_pos = start_pos + tok0;                    // the tile's first row sees the fewest keys
-  const int wave_hi = start_pos + min(tok0 + 15, q_len - 1);   // beyond it this tile has nothing to do
-  const int wave_max_lo = window > 0 ? max(0, wave_hi - window + 1) : 0;
-
-  bf16x8 qb[DSTEPS];
+  // this wave's row tiles; this lane's row (in both products) is token tok0 + col of the tile's head
+  const bool live = first_tile + wave * RT < n_row_tiles;
+  int row_pos[RT], row_lo[RT], row_tok[RT], head[RT];
+  bool row_ok[RT];
+  int wave_lo_pos = 0x7fffffff, wave_hi = -1, wave_max_lo = 0;
+  bf16x8 qb[RT][DSTEPS];
 #pragma unroll
-  for (int s = 0; s < DSTEPS; ++s) {
-    const int d = s * 32 + grp * 8;
-    qb[s] = (row_ok && d < D) ? *reinterpret_cast<const bf16x8*>(q + ((size_t)(q_begin + row_tok) * Hq + head) * D + d)
-                              : zero8();
+  for (int r = 0; r < RT; ++r) {
+    const int my_tile = first_tile + wave * RT + r;
+    const bool tile_live = my_tile < n_row_tiles;
+    head[r] = kvh * G + (tile_live ? my_tile % G : 0);
+    const int tok0 = tile_live ? (my_tile / G) * 16 : 0;
+    row_tok[r] = tok0 + col;
+    row_ok[r] = tile_live && row_tok[r] < q_len;
+    row_pos[r] = tile_live ? start_pos + min(row_tok[r], q_len - 1) : -1;    // a tile beyond the portion sees no key
+    row_lo[r] = window > 0 ? max(0, row_pos[r] - window + 1) : 0;
+    if (tile_live) {
+      const int hi = start_pos + min(tok0 + 15, q_len - 1);                 // beyond it the tile has nothing to do
+      wave_lo_pos = min(wave_lo_pos, start_pos + tok0);                       // the tile's first row sees the fewest keys
+      wave_hi = max(wave_hi, hi);
+      wave_max_lo = max(wave_max_lo, window > 0 ? max(0, hi - window + 1) : 0);
+    }
+#pragma unroll
+    for (int s = 0; s < DSTEPS; ++s) {
+      const int d = s * 32 + grp * 8;
+      qb[r][s] = (row_ok[r] && d < D)
+                     ? *reinterpret_cast<const bf16x8*>(q + ((size_t)(q_begin + row_tok[r]) * Hq + head[r]) * D + d)
+                     : zero8();
+    }
   }
-  float m_run = -INFINITY;                                 // of row `col`, the same in all four lane groups (base 2)
-  float l_part = 0.f;                                      // this lane's share of the row's sum
-  floatx4 o[DTILES];                                       // o[dt][j]: entry dt * 16 + 4 grp + j of row `col`
+  float m_run[RT], l_part[RT];                             // of row `col` (base 2); l_part is this lane's share of the row's sum
+  floatx4 o[RT][DTILES];                                   // o[r][dt][j]: entry dt * 16 + 4 grp + j of row `col`
 #pragma unroll
-  for (int dt = 0; dt < DTILES; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < RT; ++r) {
+    m_run[r] = -INFINITY;
+    l_part[r] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) o[r][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
 
   const int* bt_g = block_tables + (size_t)req * max_blocks;
   if (BT_IN_LDS) {
@@ -173,63 +192,72 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
   };
 
   auto compute = [&](int kb, const bf16_t* k_s, const bf16_t* v_s) {
-    // ---- scores of the tile's keys for this wave's 16 rows
-    floatx4 s4[KT];
+    // ---- scores of the tile's keys for this wave's rows: every K operand serves all row tiles
+    floatx4 s4[RT][KT];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-      s4[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < RT; ++r) s4[r][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < DSTEPS; ++s) {
         const int piece = s * 4 + grp;
         const bf16x8 ka = piece < CH ? *reinterpret_cast<const bf16x8*>(k_s + (kt * 16 + col) * D + (piece ^ (col & KSWZ)) * 8)
                                      : zero8();
-        s4[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[s], s4[kt], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) s4[r][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[r][s], s4[r][kt], 0, 0, 0);
       }
     }
     // tiles wholly inside every row's range need no mask
     const bool need_mask = kb + BN - 1 > wave_lo_pos || kb < wave_max_lo;
-    float m_tile = -INFINITY;
+    bf16x8 pa[RT][KT / 2];                                 // P of keys (32 a + 4 grp + j) and (32 a + 16 + 4 grp + j)
+    float alpha[RT];
+    bool grow[RT];
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt)
+    for (int r = 0; r < RT; ++r) {
+      float m_tile = -INFINITY;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float v = s4[kt][j] * scale_log2e;
-        if (need_mask) {
-          const int key = kb + kt * 16 + grp * 4 + j;
-          if (key > row_pos || key < row_lo) v = -INFINITY;
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float v = s4[r][kt][j] * scale_log2e;
+          if (need_mask) {
+            const int key = kb + kt * 16 + grp * 4 + j;
+            if (key > row_pos[r] || key < row_lo[r]) v = -INFINITY;
+          }
+          s4[r][kt][j] = v;
+          m_tile = fmaxf(m_tile, v);
         }
-        s4[kt][j] = v;
-        m_tile = fmaxf(m_tile, v);
-      }
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-    // The running maximum is only a reference point: as long as no row of the wave has grown by more than 2^6
-    // over its reference, the reference stays and the output needs no rescaling (P stays below 64).
-    const bool grow = __any(m_tile > m_run + 6.0f);
-    const float m_new = grow ? fmaxf(m_run, m_tile) : m_run;
-    const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
-    float psum = 0.f;
-    bf16x8 pa[KT / 2];                                     // P of keys (32 a + 4 grp + j) and (32 a + 16 + 4 grp + j)
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+      // The running maximum is only a reference point: as long as no row of the wave has grown by more than 2^6
+      // over its reference, the reference stays and the output needs no rescaling (P stays below 64).
+      grow[r] = __any(m_tile > m_run[r] + 6.0f);
+      const float m_new = grow[r] ? fmaxf(m_run[r], m_tile) : m_run[r];
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
+      alpha[r] = __builtin_amdgcn_exp2f(m_run[r] - m_safe);
+      float psum = 0.f;
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt)
+      for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float p = __builtin_amdgcn_exp2f(s4[kt][j] - m_safe);
-        psum += p;
-        pa[kt / 2][(kt % 2) * 4 + j] = (__bf16)p;
-      }
-    l_part = l_part * alpha + psum;
-    m_run = m_new;
+        for (int j = 0; j < 4; ++j) {
+          const float p = __builtin_amdgcn_exp2f(s4[r][kt][j] - m_safe);
+          psum += p;
+          pa[r][kt / 2][(kt % 2) * 4 + j] = (__bf16)p;
+        }
+      l_part[r] = l_part[r] * alpha[r] + psum;
+      m_run[r] = m_new;
+    }
     // this lane points at key 4 grp + col / 4 of a 16-key sub-tile, entries 4 (col % 4).. of the 16-entry block dt
     const int tr_key = grp * 4 + (col >> 2);
     const int tr_piece = (col & 3) >> 1, tr_half = (col & 1) * 4;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
-      if (grow) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
-      }
+      for (int r = 0; r < RT; ++r)
+        if (grow[r]) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o[r][dt][j] *= alpha[r];
+        }
 #pragma unroll
       for (int a = 0; a < KT / 2; ++a) {
         // this lane's eight summation slots: keys 32 a + 4 grp + (0..3) and 32 a + 16 + 4 grp + (0..3), entry dt * 16 + col
@@ -241,7 +269,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
         typedef short short8_t __attribute__((ext_vector_type(8)));
         const short8_t both = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
         const bf16x8 va = __builtin_bit_cast(bf16x8, both);
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pa[a], o[dt], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) o[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pa[r][a], o[r][dt], 0, 0, 0);
       }
     }
   };
@@ -262,18 +291,21 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
     if (live && kb + BN <= wave_hi) compute(kb + BN, k_s1, v_s1);
   }
   if (!live) return;
-  float l = l_part;
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  if (row_ok) {
-    const float inv = 1.0f / l;
-    bf16_t* dst = out + ((size_t)(q_begin + row_tok) * Hq + head) * D;
 #pragma unroll
-    for (int dt = 0; dt < DTILES; ++dt) {
-      bf16x4 four;
+  for (int r = 0; r < RT; ++r) {
+    float l = l_part[r];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (row_ok[r]) {
+      const float inv = 1.0f / l;
+      bf16_t* dst = out + ((size_t)(q_begin + row_tok[r]) * Hq + head[r]) * D;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) four[j] = (__bf16)(o[dt][j] * inv);
-      *reinterpret_cast<bf16x4*>(dst + dt * 16 + grp * 4) = four;
+      for (int dt = 0; dt < DTILES; ++dt) {
+        bf16x4 four;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) four[j] = (__bf16)(o[r][dt][j] * inv);
+        *reinterpret_cast<bf16x4*>(dst + dt * 16 + grp * 4) = four;
+      }
     }
   }
 }
@@ -293,18 +325,25 @@ extern "C" int nhv_prefill_attention_bf16(const void* q, const void* k_cache, co
     if (page_size == (1 << b)) page_shift = b;
   const int G = Hq / Hkv;
   const long long row_tiles = (long long)G * ((max_q_len + 15) / 16);
-  const long long gx = (row_tiles + prefill::TPB - 1) / prefill::TPB;
+  // two row tiles a wave where that still leaves a block for every compute unit
+  const bool two = prefill::MAX_RT >= 2 && (row_tiles + 7) / 8 * Hkv * B >= 256;
+  const int tpb = two ? 8 : 4;
+  const long long gx = (row_tiles + tpb - 1) / tpb;
   NHV_REQUIRE(gx <= 0x7fffffff && Hkv <= 65535 && B <= 65535, "prefill attention: grid too large");
-  if (max_blocks <= prefill::BT_LDS)
-    hipLaunchKernelGGL(prefill::prefill_attention_kernel<true>, dim3((unsigned)gx, Hkv, B), dim3(256), 0,
-                       (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out,
-                       (const int*)cu_seqlens_q, (const int*)context_lens, (const int*)block_tables, max_blocks, Hq, Hkv,
-                       page_size, page_shift, scale * 1.4426950408889634f, window);
-  else
-    hipLaunchKernelGGL(prefill::prefill_attention_kernel<false>, dim3((unsigned)gx, Hkv, B), dim3(256), 0,
-                       (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out,
-                       (const int*)cu_seqlens_q, (const int*)context_lens, (const int*)block_tables, max_blocks, Hq, Hkv,
-                       page_size, page_shift, scale * 1.4426950408889634f, window);
+#define NHV_PREFILL_LAUNCH(BT, RT_)                                                                                    \
+  hipLaunchKernelGGL((prefill::prefill_attention_kernel<BT, RT_>), dim3((unsigned)gx, Hkv, B), dim3(256), 0,         \
+                     (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, \
+                     (const int*)cu_seqlens_q, (const int*)context_lens, (const int*)block_tables, max_blocks, Hq, Hkv, \
+                     page_size, page_shift, scale * 1.4426950408889634f, window)
+  const bool bt_in_lds = max_blocks <= prefill::BT_LDS;
+  if (two) {
+    if (bt_in_lds) NHV_PREFILL_LAUNCH(true, prefill::MAX_RT);
+    else NHV_PREFILL_LAUNCH(false, prefill::MAX_RT);
+  } else {
+    if (bt_in_lds) NHV_PREFILL_LAUNCH(true, 1);
+    else NHV_PREFILL_LAUNCH(false, 1);
+  }
+#undef NHV_PREFILL_LAUNCH
   NHV_LAUNCH_CHECK("prefill_attention");
   return 0;
 }
