@@ -162,10 +162,13 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
         s4[kt][j] = v;
         m_tile = fmaxf(m_tile, v);
       }
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-    // the maximum is a reference point only: it moves when some head has grown by more than 2^6 over it
+    // the maximum is a reference point only: it moves when some head has grown by more than 2^6 over it, which
+    // shows in the lanes' own maxima; the head's maximum over its four lanes is only needed then
     const bool grow = __any(m_tile > m_run + 6.0f);
+    if (grow) {
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+    }
     const float m_new = grow ? fmaxf(m_run, m_tile) : m_run;     // finite: every round holds a visible key
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float psum = 0.f;

@@ -227,11 +227,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
           s4[r][kt][j] = v;
           m_tile = fmaxf(m_tile, v);
         }
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
       // The running maximum is only a reference point: as long as no row of the wave has grown by more than 2^6
-      // over its reference, the reference stays and the output needs no rescaling (P stays below 64).
+      // over its reference, the reference stays and the output needs no rescaling (P stays below 64). Whether
+      // any row has grown shows in the lanes' own maxima; the row's maximum over its four lanes is only needed then.
       grow[r] = __any(m_tile > m_run[r] + 6.0f);
+      if (grow[r]) {
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+      }
       const float m_new = grow[r] ? fmaxf(m_run[r], m_tile) : m_run[r];
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
       alpha[r] = __builtin_amdgcn_exp2f(m_run[r] - m_safe);
