@@ -214,19 +214,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     bool grow[RT];
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
+      // the scale (times log2 e) is positive: the maximum is taken of the raw scores, and the scaling rides in the
+      // multiply-add that also subtracts the reference
       float m_tile = -INFINITY;
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          float v = s4[r][kt][j] * scale_log2e;
           if (need_mask) {
             const int key = kb + kt * 16 + grp * 4 + j;
-            if (key > row_pos[r] || key < row_lo[r]) v = -INFINITY;
+            if (key > row_pos[r] || key < row_lo[r]) s4[r][kt][j] = -INFINITY;
           }
-          s4[r][kt][j] = v;
-          m_tile = fmaxf(m_tile, v);
+          m_tile = fmaxf(m_tile, s4[r][kt][j]);
         }
+      m_tile *= scale_log2e;
       // The running maximum is only a reference point: as long as no row of the wave has grown by more than 2^6
       // over its reference, the reference stays and the output needs no rescaling (P stays below 64). Whether
       // any row has grown shows in the lanes' own maxima; the row's maximum over its four lanes is only needed then.
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float p = __builtin_amdgcn_exp2f(s4[r][kt][j] - m_safe);
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s4[r][kt][j], scale_log2e, -m_safe));
           psum += p;
           pa[r][kt / 2][(kt % 2) * 4 + j] = (__bf16)p;
         }
