@@ -3,6 +3,9 @@
 // argmax_i softmax(logits / T)_i / e_i with e_i ~ Exp(1), which draws i with
 // probability softmax_i. The noise is a function of (key[row], i) only, so what a
 // request samples does not depend on its batch mates.
+// Greedy rows are cut into pieces of 4096 logits, one block each (a row of a large
+// vocabulary read by one block alone takes ten times as long); a second kernel picks
+// among the pieces' winners and does the rows with a temperature, one block a row.
 #include "nhv_common.h"
 #include <math.h>
 
@@ -52,15 +55,48 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return r;
 }
 
+constexpr int PIECE = 4096;                 // logits per block of the first kernel
+
+// the best of one piece of a greedy row; rows with a temperature are left to the second kernel
+__global__ __launch_bounds__(256) void greedy_pieces_kernel(const float* __restrict__ logits, const float* __restrict__ temperatures,
+                                                            float* __restrict__ piece_value, int* __restrict__ piece_index, int V,
+                                                            int pieces) {
+  __shared__ Best bscratch[16];
+  const int r = blockIdx.y, c = blockIdx.x;
+  if (temperatures[r] > 0.f) return;
+  const float* row = logits + (size_t)r * V;
+  const int lo = c * PIECE, hi = min(V, lo + PIECE);
+  Best best{-INFINITY, 0x7fffffff};
+  if ((((uintptr_t)row) & 15) == 0 && (V & 3) == 0) {
+    for (int i = lo + threadIdx.x * 4; i < hi; i += 256 * 4) {       // hi - lo and lo are multiples of 4
+      const float4 v = *reinterpret_cast<const float4*>(row + i);
+      best = better(best, Best{v.x, i});
+      best = better(best, Best{v.y, i + 1});
+      best = better(best, Best{v.z, i + 2});
+      best = better(best, Best{v.w, i + 3});
+    }
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += 256) best = better(best, Best{row[i], i});
+  }
+  best = block_best(best, bscratch);
+  if (threadIdx.x == 0) {
+    piece_value[(size_t)r * pieces + c] = best.v;
+    piece_index[(size_t)r * pieces + c] = best.i;
+  }
+}
+
 __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperatures,
-                                                      const uint64_t* __restrict__ keys, int* __restrict__ tokens, int V) {
+                                                      const uint64_t* __restrict__ keys, int* __restrict__ tokens, int V,
+                                                      const float* __restrict__ piece_value,
+                                                      const int* __restrict__ piece_index, int pieces) {
   __shared__ float fscratch[16];
   __shared__ Best bscratch[16];
   const float* row = logits + (size_t)blockIdx.x * V;
   const float temp = temperatures[blockIdx.x];
   Best best{-INFINITY, 0x7fffffff};
   if (temp <= 0.f) {
-    for (int i = threadIdx.x; i < V; i += blockDim.x) best = better(best, Best{row[i], i});
+    for (int c = threadIdx.x; c < pieces; c += blockDim.x)
+      best = better(best, Best{piece_value[(size_t)blockIdx.x * pieces + c], piece_index[(size_t)blockIdx.x * pieces + c]});
   } else {
     float mx = -INFINITY;
     for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, row[i] / temp);
@@ -78,12 +114,23 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   if (threadIdx.x == 0) tokens[blockIdx.x] = best.i;
 }
 
+// how many floats (and as many ints) of scratch nhv_sample needs for n rows of V logits
+extern "C" int nhv_sample_pieces(int V) { return (V + PIECE - 1) / PIECE; }
+
+// piece_value: float [n, nhv_sample_pieces(V)], piece_index: int of the same shape: scratch of this call
 extern "C" int nhv_sample(const void* logits, const void* temperatures, const void* keys, void* tokens, int n, int V,
-                          void* stream) {
+                          void* piece_value, void* piece_index, void* stream) {
   NHV_REQUIRE(n > 0 && V > 0, "sample: bad sizes n=%d V=%d", n, V);
+  NHV_REQUIRE(n <= 65535, "sample: %d rows are beyond this kernel's limit of 65535", n);
+  NHV_REQUIRE(piece_value && piece_index, "sample: no scratch");
+  const int pieces = (V + PIECE - 1) / PIECE;
+  hipLaunchKernelGGL(greedy_pieces_kernel, dim3(pieces, n), dim3(256), 0, (hipStream_t)stream, (const float*)logits,
+                     (const float*)temperatures, (float*)piece_value, (int*)piece_index, V, pieces);
+  NHV_LAUNCH_CHECK("sample (pieces)");
   const int threads = V >= 4096 ? 1024 : 256;
   hipLaunchKernelGGL(sample_kernel, dim3(n), dim3(threads), 0, (hipStream_t)stream, (const float*)logits,
-                     (const float*)temperatures, (const uint64_t*)keys, (int*)tokens, V);
+                     (const float*)temperatures, (const uint64_t*)keys, (int*)tokens, V, (const float*)piece_value,
+                     (const int*)piece_index, pieces);
   NHV_LAUNCH_CHECK("sample");
   return 0;
 }

@@ -200,7 +200,11 @@ class NativeBackend:
 
     def sample(self, logits, temperatures, keys, tokens):
         n, V = logits.shape
-        self._call("nhv_sample", _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(tokens), n, V, _stream())
+        pieces = self.lib.nhv_sample_pieces(V)
+        piece_value = torch.empty((n, pieces), dtype=torch.float32, device=logits.device)
+        piece_index = torch.empty((n, pieces), dtype=torch.int32, device=logits.device)
+        self._call("nhv_sample", _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(tokens), n, V, _ptr(piece_value),
+                   _ptr(piece_index), _stream())
 
 
 class KernelTimes:
