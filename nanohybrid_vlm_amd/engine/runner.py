@@ -156,10 +156,10 @@ class ModelRunner:
         return pages
 
     # ------------------------------------------------------------------ the step
-    def _stage(self, arrays: list[np.ndarray]) -> list[torch.Tensor]:
-        """All index arrays of a step go to the device in one copy."""
-        sizes = [a.size for a in arrays]
-        total = sum(sizes)
+    def _fill_host_buffer(self, arrays: list[np.ndarray]) -> torch.Tensor:
+        """The step's index arrays one after the other in host memory (pinned, and reused from step to step, where
+        the device is a GPU)."""
+        total = sum(a.size for a in arrays)
         if self.device.type == "cuda":
             if self._pinned is None or self._pinned.numel() < total:
                 self._pinned = torch.empty(max(total, 4096) * 2, dtype=torch.int32, pin_memory=True)
@@ -171,13 +171,23 @@ class ModelRunner:
             host = torch.empty(total, dtype=torch.int32)
         flat = host.numpy()
         offset = 0
-        for a, n in zip(arrays, sizes):
-            flat[offset:offset + n] = a.reshape(-1)
-            offset += n
-        dev = host.to(self.device, non_blocking=True)
+        for a in arrays:
+            flat[offset:offset + a.size] = a.reshape(-1)
+            offset += a.size
+        return host
+
+    def _copy_issued(self) -> None:
+        """Marks the point after which the host buffer may be written again."""
         if self.device.type == "cuda":
             self._pinned_free = torch.cuda.Event()
             self._pinned_free.record()
+
+    def _stage(self, arrays: list[np.ndarray]) -> list[torch.Tensor]:
+        """All index arrays of a step go to the device in one copy."""
+        sizes = [a.size for a in arrays]
+        host = self._fill_host_buffer(arrays)
+        dev = host.to(self.device, non_blocking=True)
+        self._copy_issued()
         out, offset = [], 0
         for a, n in zip(arrays, sizes):
             out.append(dev[offset:offset + n].view(a.shape))
@@ -198,6 +208,11 @@ class ModelRunner:
             seen.add(e.request_id)
             if len(e.tokens) == 0:
                 raise ValueError(f"request {e.request_id!r}: a step entry needs at least one token")
+        if all(len(e.tokens) == 1 for e in entries):
+            return self._layout_single_tokens(entries, pad_to, table_width)
+        return self._layout_general(entries, pad_to, table_width)
+
+    def _layout_general(self, entries: list[StepEntry], pad_to: int | None, table_width: int | None):
         cache = self.cache
         starts, new_lens = [], []
         for e in entries:
@@ -259,6 +274,59 @@ class ModelRunner:
                 "max_q_len": int(q_lens.max()), "max_context_len": int(max(new_lens))}
         return arrays, meta
 
+    def _layout_single_tokens(self, entries: list[StepEntry], pad_to: int | None, table_width: int | None):
+        """``_layout`` for a step in which every request brings one token (a decoding step): the same arrays,
+        built from plain lists (this runs between two steps, while the GPU waits)."""
+        cache = self.cache
+        B = len(entries)
+        pad = 0 if pad_to is None else pad_to - B
+        starts, ids, slots, rows = [], [], [], []
+        for i, e in enumerate(entries):
+            if e.request_id not in cache:
+                cache.admit(e.request_id)
+            start = cache.num_tokens(e.request_id)
+            if start + 1 > self.max_position:
+                raise ValueError(f"request {e.request_id!r}: {start + 1} tokens exceed the model's "
+                                 f"{self.max_position} positions")
+            token = e.tokens[0]
+            if not 0 <= token < self.vocab_size:
+                raise ValueError(f"token id {token} is outside the vocabulary of {self.vocab_size}")
+            cache.reserve(e.request_id, start + 1)
+            starts.append(start)
+            ids.append(token)
+            slots.append(cache.state_slot(e.request_id))
+            for w in e.want:
+                if w != 0:
+                    raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its 1 tokens")
+                rows.append(i)
+        n = B + pad
+        new_lens = [s + 1 for s in starts]
+        zeros = [0] * pad
+        arrays = [np.array(ids + zeros, dtype=np.int32), np.array(starts + zeros, dtype=np.int32),
+                  np.arange(n, dtype=np.int32), np.arange(n + 1, dtype=np.int32),
+                  np.array(new_lens + [1] * pad, dtype=np.int32), np.array(slots + zeros, dtype=np.int32)]
+        for gi, g in enumerate(cache.groups):
+            tables = [cache.block_table(e.request_id, gi) for e in entries]
+            width = table_width or max(1, max(len(t) for t in tables))
+            # padding rows point at page 0 (a place that exists) and store nothing (slot -1)
+            flat, slot_mapping = [], [-1] * n
+            ps = g.page_size
+            for i, t in enumerate(tables):
+                if len(t) > width:
+                    raise ValueError(f"request {entries[i].request_id!r} holds {len(t)} pages; the tables have {width}")
+                flat += t
+                flat += [NO_PAGE] * (width - len(t))
+                page = t[starts[i] // ps]
+                if page == NO_PAGE:
+                    raise RuntimeError(f"request {entries[i].request_id!r}: a new token falls on a page that was given back")
+                slot_mapping[i] = page * ps + starts[i] % ps
+            flat += ([0] + [NO_PAGE] * (width - 1)) * pad
+            bt = np.array(flat, dtype=np.int32).reshape(n, width)
+            arrays += [np.array(slot_mapping, dtype=np.int32), bt]
+        meta = {"B": n, "T": n, "rows": rows, "starts": starts, "new_lens": new_lens, "q_lens": [1] * n,
+                "state_slots": slots + zeros, "max_q_len": 1, "max_context_len": max(new_lens)}
+        return arrays, meta
+
     def _context(self, dev: list[torch.Tensor], meta: dict, logit_rows: torch.Tensor | None, num_logit_rows: int,
                  max_context_len: int) -> StepContext:
         d_ids, d_pos, d_req, d_cu, d_ctx, d_slots = dev[:6]
@@ -318,21 +386,8 @@ class ModelRunner:
         g = self._graphs.get(bucket)
         if g is None:
             g = self._graphs[bucket] = self._capture(bucket, arrays, meta, width)
-        sizes = [a.size for a in arrays]
-        total = sum(sizes)
-        if self._pinned is None or self._pinned.numel() < total:
-            self._pinned = torch.empty(max(total, 4096) * 2, dtype=torch.int32, pin_memory=True)
-            self._pinned_free = None
-        if self._pinned_free is not None:
-            self._pinned_free.synchronize()
-        flat = self._pinned[:total].numpy()
-        offset = 0
-        for a, n in zip(arrays, sizes):
-            flat[offset:offset + n] = a.reshape(-1)
-            offset += n
-        g["index"].copy_(self._pinned[:total], non_blocking=True)
-        self._pinned_free = torch.cuda.Event()
-        self._pinned_free.record()
+        g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
+        self._copy_issued()
         g["graph"].replay()
         for e, n in zip(entries, meta["new_lens"]):
             self._poison(self.cache.commit(e.request_id, n, e.tokens))
