@@ -225,7 +225,17 @@ class CacheManager:
         in_use = sum(1 for p in self.known_prefix(tokens) if p in pool.used)
         return -(-len(tokens) // g.page_size) - in_use <= pool.num_free
 
+    def _has_pages(self, rc: RequestCache, new_len: int) -> bool:
+        """Whether the request's tables already reach ``new_len`` (the usual case of a decoding step)."""
+        for g, table in zip(self.groups, rc.tables):
+            if len(table) * g.page_size < new_len:
+                return False
+        return True
+
     def can_reserve(self, request_id, new_len: int) -> bool:
+        rc = self.requests.get(request_id)
+        if rc is not None and self._has_pages(rc, new_len):
+            return True
         need = self.pages_needed(request_id, new_len)
         return all(n <= p.num_free for n, p in zip(need, self.pools))
 
@@ -278,6 +288,8 @@ class CacheManager:
         rc = self.requests[request_id]
         if new_len < rc.num_tokens:
             raise CacheError(f"request {request_id!r}: cannot shrink from {rc.num_tokens} to {new_len} tokens")
+        if self._has_pages(rc, new_len):
+            return
         need = self.pages_needed(request_id, new_len)
         for gi, n in enumerate(need):
             if n > self.pools[gi].num_free:
