@@ -6,8 +6,8 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-void nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
-                             int out_dtype, hipStream_t s);
+int nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
+                            int out_dtype, hipStream_t s);
 
 __device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x8 sk_zero8() {
@@ -158,7 +158,7 @@ extern "C" int nhv_gemm_skinny_bf16(const void* x, const void* w, const void* bi
     NHV_LAUNCH_CHECK("gemm_mid_bf16");
     return 0;
   }
-  nhv_gemm_fewrows_launch(false, x, w, bias, y, M, N, K, out_dtype, s);
+  if (nhv_gemm_fewrows_launch(false, x, w, bias, y, M, N, K, out_dtype, s)) return 1;
   NHV_LAUNCH_CHECK("gemm_fewrows_bf16");
   return 0;
 }
@@ -173,7 +173,7 @@ extern "C" int nhv_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, i
     NHV_LAUNCH_CHECK("gemm_mid_glu_bf16");
     return 0;
   }
-  nhv_gemm_fewrows_launch(true, x, w, nullptr, y, M, N, K, out_dtype, s);
+  if (nhv_gemm_fewrows_launch(true, x, w, nullptr, y, M, N, K, out_dtype, s)) return 1;
   NHV_LAUNCH_CHECK("gemm_fewrows_glu_bf16");
   return 0;
 }
