@@ -119,35 +119,25 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_kernel(const bf16_t* 
 typedef __attribute__((address_space(3))) void* lds_ptr;
 typedef const __attribute__((address_space(1))) void* global_ptr;
 
-// The kernel with x resident in LDS: x_s[m][K + 8] (the 16 bytes between rows spread the rows over the
+// The kernel with x resident in LDS: x_s[m][columns + 8] (the 16 bytes between rows spread the rows over the
 // banks), then for tile = blockIdx.x, + gridDim.x, ...: waves split K as above, sums meet in one of two
 // LDS buffers (one barrier a tile), and the waves take turns in adding them up and writing the result.
+// Where all of x is too much for LDS and every block has one tile only, x comes in `nchunks` pieces of
+// `chunk_steps` steps of 32 columns, one after the other, and the sums run on over the pieces.
+// (Asking for the next tile's first loads before a tile's sums are exchanged was measured and changed nothing.)
 template <int WAVES, int UNROLL, bool GLU, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                            const bf16_t* __restrict__ bias, TOut* __restrict__ y,
-                                                                           int M, int N, int K, int tiles, int steps_per_wave) {
+                                                                           int M, int N, int K, int tiles, int nchunks,
+                                                                           int chunk_steps, int steps_per_wave) {
   constexpr int NA = GLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float(*red)[NA][4][64] = reinterpret_cast<float(*)[NA][4][64]>(lds_raw);      // [2 WAVES][NA][4][64]
   bf16_t* x_s = reinterpret_cast<bf16_t*>(lds_raw + 2 * WAVES * NA * 4 * 64 * sizeof(float));
-  const int pitch = K + 8;
+  const int pitch = min(K, chunk_steps * 32) + 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  // x into LDS: a wave's load brings 64 consecutive 16-byte pieces of one row
-  const int pieces_per_row = K / 8;
-  const int loads_per_row = (pieces_per_row + 63) / 64;
-  for (int job = wave; job < M * loads_per_row; job += WAVES) {
-    const int m = job / loads_per_row, part = job % loads_per_row;
-    const int piece = part * 64 + lane;
-    if (piece < pieces_per_row)
-      __builtin_amdgcn_global_load_lds((global_ptr)(x + (size_t)m * K + piece * 8), (lds_ptr)(x_s + m * pitch + part * 512), 16, 0, 0);
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
   const int ksteps = (K + 31) / 32;
-  const int first = wave * steps_per_wave;
-  const int last = min(first + steps_per_wave, ksteps);
   const bool m_ok = col < M;
   const bf16_t* xrow_s = x_s + (m_ok ? col : 0) * pitch;
   int parity = 0, turn = 0;
@@ -160,22 +150,43 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
     floatx4 acc[NA];
 #pragma unroll
     for (int na = 0; na < NA; ++na) acc[na] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int s0 = first; s0 < last; s0 += UNROLL) {
-      bf16x8 a[UNROLL][NA];
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const int k = (s0 + u) * 32 + grp * 8;
-        const bool k_ok = (s0 + u < last) && k < K;
-#pragma unroll
-        for (int na = 0; na < NA; ++na) a[u][na] = (n_ok && k_ok) ? load8(wrow[na] + k) : zero8();
+    for (int c = 0; c < nchunks; ++c) {
+      const int c0 = c * chunk_steps, c_end = min(c0 + chunk_steps, ksteps);
+      if (nchunks > 1 || tile == (int)blockIdx.x) {
+        // this piece of x into LDS: a wave's load brings 64 consecutive 16-byte pieces of one row
+        if (c > 0) __syncthreads();                      // the piece before has been read by every wave
+        const int col0 = c0 * 32;
+        const int pieces_per_row = (min(K, c_end * 32) - col0) / 8;
+        const int loads_per_row = (pieces_per_row + 63) / 64;
+        for (int job = wave; job < M * loads_per_row; job += WAVES) {
+          const int m = job / loads_per_row, part = job % loads_per_row;
+          const int piece = part * 64 + lane;
+          if (piece < pieces_per_row)
+            __builtin_amdgcn_global_load_lds((global_ptr)(x + (size_t)m * K + col0 + piece * 8),
+                                             (lds_ptr)(x_s + m * pitch + part * 512), 16, 0, 0);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
       }
+      const int first = c0 + wave * steps_per_wave;
+      const int last = min(first + steps_per_wave, c_end);
+      for (int s0 = first; s0 < last; s0 += UNROLL) {
+        bf16x8 a[UNROLL][NA];
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const int k = (s0 + u) * 32 + grp * 8;
-        const bool k_ok = (s0 + u < last) && k < K;
-        const bf16x8 b = (m_ok && k_ok) ? *reinterpret_cast<const bf16x8*>(xrow_s + k) : zero8();
+        for (int u = 0; u < UNROLL; ++u) {
+          const int k = (s0 + u) * 32 + grp * 8;
+          const bool k_ok = (s0 + u < last) && k < K;
 #pragma unroll
-        for (int na = 0; na < NA; ++na) acc[na] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][na], b, acc[na], 0, 0, 0);
+          for (int na = 0; na < NA; ++na) a[u][na] = (n_ok && k_ok) ? load8(wrow[na] + k) : zero8();
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const int k = (s0 + u) * 32 + grp * 8;
+          const bool k_ok = (s0 + u < last) && k < K;
+          const bf16x8 b = (m_ok && k_ok) ? *reinterpret_cast<const bf16x8*>(xrow_s + (k - c0 * 32)) : zero8();
+#pragma unroll
+          for (int na = 0; na < NA; ++na) acc[na] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][na], b, acc[na], 0, 0, 0);
+        }
       }
     }
     float(*my_red)[NA][4][64] = red + parity * WAVES;
@@ -211,15 +222,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
 constexpr size_t LDS_BYTES = 160 * 1024;
 
 // The resident kernel's shape: waves, loads in flight and blocks per compute unit, from the best variants measured
-// (same shapes as below); waves == 0 when x does not fit.
+// (same shapes as below), and in how many pieces x comes; waves == 0 when this kernel is not the one to take.
 struct ResidentPlan {
-  int waves, unroll, blocks_per_cu;
+  int waves, unroll, blocks_per_cu, nchunks, chunk_steps;
   size_t lds;
 };
 static ResidentPlan resident_plan(bool glu, int M, int N, int K) {
-  const size_t x_bytes = (size_t)M * (K + 8) * 2;
-  auto lds_of = [&](int waves) { return (size_t)2 * waves * (glu ? 2 : 1) * 4 * 64 * sizeof(float) + x_bytes; };
-  const int tiles = (N + 15) / 16;
+  const int tiles = (N + 15) / 16, ksteps = (K + 31) / 32;
+  auto lds_of = [&](int waves, int steps) {
+    const int columns = steps * 32 < K ? steps * 32 : K;
+    return (size_t)2 * waves * (glu ? 2 : 1) * 4 * 64 * sizeof(float) + (size_t)M * (columns + 8) * 2;
+  };
   int waves, unroll;
   if (glu) {
     waves = M <= 12 ? 8 : 4;
@@ -231,18 +244,33 @@ static ResidentPlan resident_plan(bool glu, int M, int N, int K) {
   } else {
     waves = 8, unroll = 2;
   }
-  if (lds_of(waves) > LDS_BYTES) {              // fewer waves need less room for their sums
-    waves = glu ? 4 : 8, unroll = 8;
-    if (lds_of(waves) > LDS_BYTES) return {0, 0, 0, 0};
+  int nchunks = 1, chunk_steps = ksteps;
+  if (lds_of(waves, ksteps) > LDS_BYTES) {      // fewer waves need less room for their sums
+    const int fewer = glu ? 4 : 8;
+    if (lds_of(fewer, ksteps) <= LDS_BYTES) {
+      waves = fewer, unroll = 8;
+    } else {
+      // x in pieces: only where every block has one tile (the pieces would come again for every tile), and
+      // pieces small enough that all blocks are on the chip at once
+      if (glu || tiles > 512) return {0, 0, 0, 0, 0, 0};
+      const int want_bpc = tiles > 256 ? 2 : 1;
+      for (nchunks = 2; nchunks <= 16; ++nchunks) {
+        chunk_steps = 2 * waves * ((ksteps + 2 * waves * nchunks - 1) / (2 * waves * nchunks));   // every wave whole lines
+        if (lds_of(waves, chunk_steps) * want_bpc <= LDS_BYTES) break;
+      }
+      if (nchunks > 16) return {0, 0, 0, 0, 0, 0};
+      nchunks = (ksteps + chunk_steps - 1) / chunk_steps;
+    }
   }
-  if (!glu && waves == 8 && unroll == 2 && 2 * lds_of(8) > LDS_BYTES) {
+  if (!glu && waves == 8 && unroll == 2 && 2 * lds_of(8, chunk_steps) > LDS_BYTES) {
     // one block a compute unit: eight waves with two loads each are too little in flight
-    if (lds_of(16) <= LDS_BYTES) waves = 16;
+    if (lds_of(16, chunk_steps) <= LDS_BYTES) waves = 16;
     else unroll = 8;
   }
-  const int by_lds = (int)(LDS_BYTES / lds_of(waves)), by_waves = 32 / waves;
+  const size_t lds = lds_of(waves, chunk_steps);
+  const int by_lds = (int)(LDS_BYTES / lds), by_waves = 32 / waves;
   const int bpc = by_lds < by_waves ? by_lds : by_waves;
-  return {waves, unroll, bpc < 2 ? 1 : 2, lds_of(waves)};
+  return {waves, unroll, bpc < 2 ? 1 : 2, nchunks, chunk_steps, lds};
 }
 
 template <int WAVES, int UNROLL, bool GLU, typename TOut>
@@ -253,12 +281,11 @@ static int launch_resident(const ResidentPlan& p, hipStream_t s, const void* x, 
   static const hipError_t allowed =
       hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
   if (allowed != hipSuccess) return nhv_fail("few-rows gemm: %s", hipGetErrorString(allowed));
-  const int ksteps = (K + 31) / 32;
-  const int steps_per_wave = 2 * ((ksteps + 2 * WAVES - 1) / (2 * WAVES));
+  const int steps_per_wave = 2 * ((p.chunk_steps + 2 * WAVES - 1) / (2 * WAVES));
   const int tiles = (N + 15) / 16;
-  const int grid = tiles < 256 * p.blocks_per_cu ? tiles : 256 * p.blocks_per_cu;
+  const int grid = (p.nchunks > 1 || tiles < 256 * p.blocks_per_cu) ? tiles : 256 * p.blocks_per_cu;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * WAVES), p.lds, s, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias,
-                     (TOut*)y, M, N, K, tiles, steps_per_wave);
+                     (TOut*)y, M, N, K, tiles, p.nchunks, p.chunk_steps, steps_per_wave);
   return 0;
 }
 
