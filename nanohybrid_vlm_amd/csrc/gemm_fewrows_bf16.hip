@@ -119,25 +119,36 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_kernel(const bf16_t* 
 typedef __attribute__((address_space(3))) void* lds_ptr;
 typedef const __attribute__((address_space(1))) void* global_ptr;
 
-// The kernel with x resident in LDS: x_s[m][columns + 8] (the 16 bytes between rows spread the rows over the
+// The kernel with x resident in LDS: x_s[m][K + 8] (the 16 bytes between rows spread the rows over the
 // banks), then for tile = blockIdx.x, + gridDim.x, ...: waves split K as above, sums meet in one of two
 // LDS buffers (one barrier a tile), and the waves take turns in adding them up and writing the result.
-// Where all of x is too much for LDS and every block has one tile only, x comes in `nchunks` pieces of
-// `chunk_steps` steps of 32 columns, one after the other, and the sums run on over the pieces.
 // (Asking for the next tile's first loads before a tile's sums are exchanged was measured and changed nothing.)
 template <int WAVES, int UNROLL, bool GLU, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                            const bf16_t* __restrict__ bias, TOut* __restrict__ y,
-                                                                           int M, int N, int K, int tiles, int nchunks,
-                                                                           int chunk_steps, int steps_per_wave) {
+                                                                           int M, int N, int K, int tiles, int steps_per_wave) {
   constexpr int NA = GLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float(*red)[NA][4][64] = reinterpret_cast<float(*)[NA][4][64]>(lds_raw);      // [2 WAVES][NA][4][64]
   bf16_t* x_s = reinterpret_cast<bf16_t*>(lds_raw + 2 * WAVES * NA * 4 * 64 * sizeof(float));
-  const int pitch = min(K, chunk_steps * 32) + 8;
+  const int pitch = K + 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
+  // x into LDS: a wave's load brings 64 consecutive 16-byte pieces of one row
+  const int pieces_per_row = K / 8;
+  const int loads_per_row = (pieces_per_row + 63) / 64;
+  for (int job = wave; job < M * loads_per_row; job += WAVES) {
+    const int m = job / loads_per_row, part = job % loads_per_row;
+    const int piece = part * 64 + lane;
+    if (piece < pieces_per_row)
+      __builtin_amdgcn_global_load_lds((global_ptr)(x + (size_t)m * K + piece * 8), (lds_ptr)(x_s + m * pitch + part * 512), 16, 0, 0);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
   const int ksteps = (K + 31) / 32;
+  const int first = wave * steps_per_wave;
+  const int last = min(first + steps_per_wave, ksteps);
   const bool m_ok = col < M;
   const bf16_t* xrow_s = x_s + (m_ok ? col : 0) * pitch;
   int parity = 0, turn = 0;
@@ -150,24 +161,102 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
     floatx4 acc[NA];
 #pragma unroll
     for (int na = 0; na < NA; ++na) acc[na] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = first; s0 < last; s0 += UNROLL) {
+      bf16x8 a[UNROLL][NA];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int k = (s0 + u) * 32 + grp * 8;
+        const bool k_ok = (s0 + u < last) && k < K;
+#pragma unroll
+        for (int na = 0; na < NA; ++na) a[u][na] = (n_ok && k_ok) ? load8(wrow[na] + k) : zero8();
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int k = (s0 + u) * 32 + grp * 8;
+        const bool k_ok = (s0 + u < last) && k < K;
+        const bf16x8 b = (m_ok && k_ok) ? *reinterpret_cast<const bf16x8*>(xrow_s + k) : zero8();
+#pragma unroll
+        for (int na = 0; na < NA; ++na) acc[na] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][na], b, acc[na], 0, 0, 0);
+      }
+    }
+    float(*my_red)[NA][4][64] = red + parity * WAVES;
+#pragma unroll
+    for (int na = 0; na < NA; ++na)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) my_red[wave][na][j][lane] = acc[na][j];
+    __syncthreads();                          // the other buffer is the one written in the next tile
+    if (wave != turn) continue;
+    float v[NA][4];
+#pragma unroll
+    for (int na = 0; na < NA; ++na)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float sum = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; ++wv) sum += my_red[wv][na][j][lane];
+        v[na][j] = sum;
+      }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + grp * 4 + j;
+      if (col < M && n < N) {
+        float r = v[0][j];
+        if (bias) r += (float)bias[n];
+        if (GLU) r = r / (1.0f + expf(-r)) * v[NA - 1][j];
+        y[(size_t)col * N + n] = (TOut)r;
+      }
+    }
+  }
+}
+
+// Where all of x is too much for LDS: the same with one tile a block and x coming in `nchunks` pieces of
+// `chunk_steps` steps of 32 columns, one after the other; the sums run on over the pieces. (A kernel of its own:
+// as an option of the one above it cost that one 4 % of its speed.)
+template <int WAVES, int UNROLL, typename TOut>
+__global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                           const bf16_t* __restrict__ bias, TOut* __restrict__ y,
+                                                                           int M, int N, int K, int tiles, int nchunks,
+                                                                           int chunk_steps, int steps_per_wave) {
+  constexpr int NA = 1;
+  constexpr bool GLU = false;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  float(*red)[NA][4][64] = reinterpret_cast<float(*)[NA][4][64]>(lds_raw);      // [2 WAVES][NA][4][64]
+  bf16_t* x_s = reinterpret_cast<bf16_t*>(lds_raw + 2 * WAVES * NA * 4 * 64 * sizeof(float));
+  const int pitch = min(K, chunk_steps * 32) + 8;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int ksteps = (K + 31) / 32;
+  const bool m_ok = col < M;
+  const bf16_t* xrow_s = x_s + (m_ok ? col : 0) * pitch;
+  // columns [32 c0, 32 c_end) of x into LDS: a wave's load brings 64 consecutive 16-byte pieces of one row
+  auto load_x = [&](int c0, int c_end) {
+    const int col0 = c0 * 32;
+    const int pieces_per_row = (min(K, c_end * 32) - col0) / 8;
+    const int loads_per_row = (pieces_per_row + 63) / 64;
+    for (int job = wave; job < M * loads_per_row; job += WAVES) {
+      const int m = job / loads_per_row, part = job % loads_per_row;
+      const int piece = part * 64 + lane;
+      if (piece < pieces_per_row)
+        __builtin_amdgcn_global_load_lds((global_ptr)(x + (size_t)m * K + col0 + piece * 8),
+                                         (lds_ptr)(x_s + m * pitch + part * 512), 16, 0, 0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+  int parity = 0, turn = 0;
+  for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x, parity ^= 1, turn = turn + 1 == WAVES ? 0 : turn + 1) {
+    const int n0 = tile * 16;
+    const bool n_ok = n0 + col < N;
+    const bf16_t* wrow[NA];
+#pragma unroll
+    for (int na = 0; na < NA; ++na) wrow[na] = w + ((size_t)na * N + (n_ok ? n0 + col : 0)) * K;
+    floatx4 acc[NA];
+#pragma unroll
+    for (int na = 0; na < NA; ++na) acc[na] = floatx4{0.f, 0.f, 0.f, 0.f};
     for (int c = 0; c < nchunks; ++c) {
       const int c0 = c * chunk_steps, c_end = min(c0 + chunk_steps, ksteps);
-      if (nchunks > 1 || tile == (int)blockIdx.x) {
-        // this piece of x into LDS: a wave's load brings 64 consecutive 16-byte pieces of one row
-        if (c > 0) __syncthreads();                      // the piece before has been read by every wave
-        const int col0 = c0 * 32;
-        const int pieces_per_row = (min(K, c_end * 32) - col0) / 8;
-        const int loads_per_row = (pieces_per_row + 63) / 64;
-        for (int job = wave; job < M * loads_per_row; job += WAVES) {
-          const int m = job / loads_per_row, part = job % loads_per_row;
-          const int piece = part * 64 + lane;
-          if (piece < pieces_per_row)
-            __builtin_amdgcn_global_load_lds((global_ptr)(x + (size_t)m * K + col0 + piece * 8),
-                                             (lds_ptr)(x_s + m * pitch + part * 512), 16, 0, 0);
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-      }
+      if (c > 0) __syncthreads();                        // the piece before has been read by every wave
+      load_x(c0, c_end);
       const int first = c0 + wave * steps_per_wave;
       const int last = min(first + steps_per_wave, c_end);
       for (int s0 = first; s0 < last; s0 += UNROLL) {
@@ -250,13 +339,12 @@ static ResidentPlan resident_plan(bool glu, int M, int N, int K) {
     if (lds_of(fewer, ksteps) <= LDS_BYTES) {
       waves = fewer, unroll = 8;
     } else {
-      // x in pieces: only where every block has one tile (the pieces would come again for every tile), and
-      // pieces small enough that all blocks are on the chip at once
-      if (glu || tiles > 512) return {0, 0, 0, 0, 0, 0};
-      const int want_bpc = tiles > 256 ? 2 : 1;
+      // x in pieces: only where every block has one tile (the pieces would come again for every tile) and all
+      // blocks are on the chip at once, one a compute unit (with 320 tiles it was measured slower by a quarter)
+      if (glu || tiles > 256) return {0, 0, 0, 0, 0, 0};
       for (nchunks = 2; nchunks <= 16; ++nchunks) {
         chunk_steps = 2 * waves * ((ksteps + 2 * waves * nchunks - 1) / (2 * waves * nchunks));   // every wave whole lines
-        if (lds_of(waves, chunk_steps) * want_bpc <= LDS_BYTES) break;
+        if (lds_of(waves, chunk_steps) <= LDS_BYTES) break;
       }
       if (nchunks > 16) return {0, 0, 0, 0, 0, 0};
       nchunks = (ksteps + chunk_steps - 1) / chunk_steps;
@@ -273,19 +361,29 @@ static ResidentPlan resident_plan(bool glu, int M, int N, int K) {
   return {waves, unroll, bpc < 2 ? 1 : 2, nchunks, chunk_steps, lds};
 }
 
-template <int WAVES, int UNROLL, bool GLU, typename TOut>
+template <int WAVES, int UNROLL, bool GLU, bool PIECES, typename TOut>
 static int launch_resident(const ResidentPlan& p, hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M,
                            int N, int K) {
-  auto kernel = gemm_fewrows_resident_kernel<WAVES, UNROLL, GLU, TOut>;
-  // more than 64 KB of dynamic LDS has to be allowed once per kernel (and per process)
-  static const hipError_t allowed =
-      hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
-  if (allowed != hipSuccess) return nhv_fail("few-rows gemm: %s", hipGetErrorString(allowed));
+  static_assert(!(GLU && PIECES), "x in pieces is not built for the gated kernel");
   const int steps_per_wave = 2 * ((p.chunk_steps + 2 * WAVES - 1) / (2 * WAVES));
   const int tiles = (N + 15) / 16;
-  const int grid = (p.nchunks > 1 || tiles < 256 * p.blocks_per_cu) ? tiles : 256 * p.blocks_per_cu;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * WAVES), p.lds, s, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias,
-                     (TOut*)y, M, N, K, tiles, p.nchunks, p.chunk_steps, steps_per_wave);
+  if constexpr (PIECES) {
+    auto kernel = gemm_fewrows_pieces_kernel<WAVES, UNROLL, TOut>;
+    // more than 64 KB of dynamic LDS has to be allowed once per kernel (and per process)
+    static const hipError_t allowed =
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
+    if (allowed != hipSuccess) return nhv_fail("few-rows gemm: %s", hipGetErrorString(allowed));
+    hipLaunchKernelGGL(kernel, dim3(tiles), dim3(64 * WAVES), p.lds, s, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias,
+                       (TOut*)y, M, N, K, tiles, p.nchunks, p.chunk_steps, steps_per_wave);
+  } else {
+    auto kernel = gemm_fewrows_resident_kernel<WAVES, UNROLL, GLU, TOut>;
+    static const hipError_t allowed =
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
+    if (allowed != hipSuccess) return nhv_fail("few-rows gemm: %s", hipGetErrorString(allowed));
+    const int grid = tiles < 256 * p.blocks_per_cu ? tiles : 256 * p.blocks_per_cu;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * WAVES), p.lds, s, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias,
+                       (TOut*)y, M, N, K, tiles, steps_per_wave);
+  }
   return 0;
 }
 
@@ -339,16 +437,19 @@ int nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* 
                             int out_dtype, hipStream_t s) {
   using namespace fewrows;
   const ResidentPlan rp = resident_plan(glu, M, N, K);
-#define NHV_RESIDENT_CASE(WV_, UN_, GLU_)                                                                         \
-  if (rp.waves == WV_ && rp.unroll == UN_ && glu == GLU_)                                                        \
-    return out_dtype == NHV_BF16 ? launch_resident<WV_, UN_, GLU_, bf16_t>(rp, s, x, w, bias, y, M, N, K)        \
-                                 : launch_resident<WV_, UN_, GLU_, float>(rp, s, x, w, bias, y, M, N, K);
-  NHV_RESIDENT_CASE(8, 2, true)
-  NHV_RESIDENT_CASE(4, 8, true)
-  NHV_RESIDENT_CASE(16, 2, false)
-  NHV_RESIDENT_CASE(8, 2, false)
-  NHV_RESIDENT_CASE(8, 8, false)
-  NHV_RESIDENT_CASE(4, 8, false)
+#define NHV_RESIDENT_CASE(WV_, UN_, GLU_, PIECES_)                                                                     \
+  if (rp.waves == WV_ && rp.unroll == UN_ && glu == GLU_ && (rp.nchunks > 1) == PIECES_)                              \
+    return out_dtype == NHV_BF16 ? launch_resident<WV_, UN_, GLU_, PIECES_, bf16_t>(rp, s, x, w, bias, y, M, N, K)    \
+                                 : launch_resident<WV_, UN_, GLU_, PIECES_, float>(rp, s, x, w, bias, y, M, N, K);
+  NHV_RESIDENT_CASE(8, 2, true, false)
+  NHV_RESIDENT_CASE(4, 8, true, false)
+  NHV_RESIDENT_CASE(16, 2, false, false)
+  NHV_RESIDENT_CASE(8, 2, false, false)
+  NHV_RESIDENT_CASE(8, 8, false, false)
+  NHV_RESIDENT_CASE(4, 8, false, false)
+  NHV_RESIDENT_CASE(16, 2, false, true)
+  NHV_RESIDENT_CASE(8, 2, false, true)
+  NHV_RESIDENT_CASE(8, 8, false, true)
 #undef NHV_RESIDENT_CASE
   const Plan p = plan(glu, M, N, K);
 #define NHV_FEWROWS_CASE(NT_, WV_, UN_, GLU_)                                              \

@@ -138,6 +138,8 @@ def test_skinny_linear_bfloat16(ops, M, N, K):
     # every way the kernel for up to 16 rows cuts the work: one or two tiles of 16 outputs per block, 4 or 8 waves
     (1, 6144, 264), (2, 5000, 4096), (5, 7168, 72), (8, 6100, 1032), (12, 5120, 520), (16, 151936, 64), (9, 10240, 40),
     (16, 16, 8), (3, 17, 25608),
+    # x too large for LDS at once, up to 256 tiles: it comes in pieces
+    (16, 4000, 12296), (7, 272, 12288), (11, 4096, 25600),
 ])
 def test_few_rows_linear_bfloat16_in_all_its_variants(ops, M, N, K):
     x = rnd(M, K, dtype=torch.bfloat16, seed=34)
