@@ -35,6 +35,7 @@ def parse_args():
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 runs")
     ap.add_argument("--eager", action="store_true", help="no HIP graphs")
+    ap.add_argument("--max-graph-batch", type=int, default=None, help="largest decode batch that replays a graph")
     return ap.parse_args()
 
 
@@ -60,7 +61,7 @@ def build_llm(args, max_seqs):
               kvcache_block_size=args.block_size, num_kvcache_blocks=max_seqs * pages_per_seq + 1,
               max_num_seqs=max_seqs, max_num_batched_tokens=max(2048, max_seqs), max_model_len=args.context,
               scheduler_policy="prefill_first",     # while prompts are fed nothing decodes, so all requests decode in step
-              enforce_eager=args.eager)
+              enforce_eager=args.eager, **({"max_graph_batch": args.max_graph_batch} if args.max_graph_batch else {}))
     return llm, cfg, full_layers
 
 

@@ -23,6 +23,7 @@ class EngineConfig:
     max_model_len: int = 4096                   # capped by max_position_embeddings
     gpu_memory_utilization: float = 0.9
     enforce_eager: bool = False                 # True: no HIP graphs for decode
+    max_graph_batch: int = 64                   # decode steps of up to this many requests replay a graph
     eos: int = -1                               # filled from config.json when -1
     kvcache_block_size: int = 256               # tokens in a page (any positive number)
     num_kvcache_blocks: int = -1                # -1: sized from free memory

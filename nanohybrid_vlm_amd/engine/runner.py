@@ -15,6 +15,7 @@ have the same meaning here.
 """
 from __future__ import annotations
 
+import sys
 from dataclasses import dataclass, field
 from typing import Hashable
 
@@ -46,7 +47,7 @@ class ModelRunner:
     def __init__(self, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 256,
                  num_pages: int | None = None, num_state_slots: int = 512, gpu_memory_utilization: float = 0.9,
                  max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None, use_graphs: bool = False,
-                 max_model_len: int | None = None, max_graph_batch: int = 16, poison_freed_pages: bool = False,
+                 max_model_len: int | None = None, max_graph_batch: int = 64, poison_freed_pages: bool = False,
                  share_prefixes: bool = False):
         """``model``/``arch``/``cfg`` may be given ready-made (weights already bound)
         instead of being read from ``model_dir``."""
@@ -76,13 +77,16 @@ class ModelRunner:
         # request no longer owns shows up in its logits
         self.poison_freed_pages = poison_freed_pages
         # decode-only steps replay a HIP graph per batch-size bucket (the reference captures CUDA graphs for
-        # the same batch sizes, nanovllm/engine/model_runner.py:2559-2594). Up to 16 requests a step is bound
-        # by launches and by the own few-rows kernels; larger batches run eagerly, where the matrix products
-        # of 17 and more rows are the library's (measured faster than the own kernel at those sizes)
+        # the same batch sizes, nanovllm/engine/model_runner.py:2559-2594). Up to 16 requests the graph holds
+        # own kernels only. Larger buckets hold the library's matrix products too (measured faster than the own
+        # kernel from 17 rows on), and a step of 17 to 48 requests is bound by its launches when run eagerly
+        # (8.3 ms at every size). A graph with a library call in it is checked when it is recorded: replayed
+        # three times, with eager work and waits between, and compared bit by bit with the eager result;
+        # a bucket whose graph fails runs eagerly from then on.
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
         self.max_model_len = min(max_model_len or self.max_position, self.max_position)
         self.max_graph_batch = max_graph_batch
-        self._graphs: dict[int, dict] = {}
+        self._graphs: dict[int, dict | None] = {}     # None: the bucket's graph failed its check
 
     # ------------------------------------------------------------------ cache
     def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens):
@@ -355,7 +359,11 @@ class ModelRunner:
         entries and of each entry's ``want`` (None if nothing is wanted)."""
         if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)
                 and not self.state_pools):
-            return self._graph_step(entries)
+            bucket = 1
+            while bucket < len(entries):
+                bucket *= 2
+            if self._graphs.get(bucket, ...) is not None:
+                return self._graph_step(entries, bucket)
         ctx, new_lens = self.build_context(entries)
         hidden = self.model.forward(ctx)
         logits = self.model.logits(hidden) if hidden is not None else None
@@ -373,22 +381,22 @@ class ModelRunner:
                 view.v[pages] = float("nan")
 
     # ------------------------------------------------------------------ decode steps as HIP graphs
-    def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor | None:
-        """A step of single tokens: the batch is padded to a bucket, written into the bucket's fixed index
+    def _graph_step(self, entries: list[StepEntry], bucket: int) -> torch.Tensor | None:
+        """A step of single tokens: the batch is padded to the bucket, written into the bucket's fixed index
         buffer, and the bucket's graph (embedding to logits of every row) is replayed."""
-        bucket = 1
-        while bucket < len(entries):
-            bucket *= 2
         width = -(-self.max_model_len // self.page_size)
         arrays, meta = self._layout(entries, pad_to=bucket, table_width=width)
         if meta["max_context_len"] > width * self.page_size:
             raise ValueError(f"a request of {meta['max_context_len']} tokens exceeds max_model_len {self.max_model_len}")
         g = self._graphs.get(bucket)
         if g is None:
-            g = self._graphs[bucket] = self._capture(bucket, arrays, meta, width)
-        g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
-        self._copy_issued()
-        g["graph"].replay()
+            g = self._capture(bucket, arrays, meta, width)
+            self._graphs[bucket] = g if g["graph"] is not None else None
+        if g["graph"] is not None:
+            g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
+            self._copy_issued()
+            g["graph"].replay()
+        # (a graph that failed its check leaves the eager result of this very step in g["logits"])
         for e, n in zip(entries, meta["new_lens"]):
             self._poison(self.cache.commit(e.request_id, n, e.tokens))
         rows = meta["rows"]
@@ -400,7 +408,7 @@ class ModelRunner:
 
     def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int) -> dict:
         """Runs the bucket's step once eagerly on its fixed buffers (so that every kernel library is loaded
-        and the allocator is warm), then records it."""
+        and the allocator is warm), then records it, and checks the graph if a library call went into it."""
         from ..native import ops
         sizes = [a.size for a in arrays]
         index = torch.zeros(sum(sizes), dtype=torch.int32, device=self.device)
@@ -413,16 +421,30 @@ class ModelRunner:
         all_rows = torch.arange(bucket, dtype=torch.int32, device=self.device)
         ctx = self._context(dev, meta, all_rows, bucket, max_context_len=width * self.page_size)
         backend = ops.backend()
-        old = getattr(backend, "own_kernels_only", False)
-        backend.own_kernels_only = True                     # nothing of a library is recorded into the graph
+        with_library = bucket > getattr(backend, "few_rows", bucket) and self.dtype == torch.bfloat16
+        old = (getattr(backend, "own_kernels_only", False), getattr(backend, "recording_graph", False))
+        backend.own_kernels_only = not with_library
+        backend.recording_graph = True                      # lengths are only bounded: kernels plan for the bound
         try:
-            self.model.logits(self.model.forward(ctx))       # warm-up; it writes the same cache slots as the replay will
+            # warm-up; it writes the same cache slots as every replay will
+            eager = self.model.logits(self.model.forward(ctx)).clone()
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.logits(self.model.forward(ctx))
+            if with_library:
+                for _ in range(3):
+                    logits.fill_(float("nan"))
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    if not torch.equal(logits, eager):
+                        print(f"[nanohybrid_vlm_amd] the graph for {bucket} requests differs from the eager step when "
+                              "replayed; steps of this size run eagerly", file=sys.stderr, flush=True)
+                        return {"graph": None, "index": index, "logits": eager, "ctx": ctx}
+                    self.model.logits(self.model.forward(ctx))      # eager work between the replays
+                    torch.cuda.synchronize()
         finally:
-            backend.own_kernels_only = old
+            backend.own_kernels_only, backend.recording_graph = old
         return {"graph": graph, "index": index, "logits": logits, "ctx": ctx}
 
     def get_memory_stats(self) -> dict:
@@ -444,7 +466,8 @@ class ModelRunner:
             "live_requests": len(self.cache.requests),
             "prefix_cache": {"enabled": self.cache.share_prefixes, "known_pages": len(self.cache.page_of_hash),
                              "shared_tokens": self.cache.num_shared_tokens},
-            "graphs_recorded": sorted(self._graphs),
+            "graphs_recorded": sorted(b for b, g in self._graphs.items() if g is not None),
+            "graphs_refused": sorted(b for b, g in self._graphs.items() if g is None),
         }
         if self.device.type == "cuda":
             free, total = torch.cuda.mem_get_info(self.device)

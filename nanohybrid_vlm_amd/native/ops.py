@@ -78,7 +78,9 @@ class NativeBackend:
 
     name = "hip"
     device_type = "cuda"
-    own_kernels_only = False      # True while a HIP graph is recorded: no library call goes into a graph
+    few_rows = 16                 # up to this many rows the own matrix kernels are the faster ones
+    own_kernels_only = False      # True: no library call (matrix products of up to 64 rows take the own kernels)
+    recording_graph = False       # True while a HIP graph is recorded: lengths are bounds, not the step's own
 
     def __init__(self):
         if not torch.cuda.is_available():
@@ -150,7 +152,7 @@ class NativeBackend:
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
         # inside a graph the lengths are only bounded (by max_model_len): plan for half the bound
-        span = batch.max_context_len // 2 if self.own_kernels_only else batch.max_context_len
+        span = batch.max_context_len // 2 if self.recording_graph else batch.max_context_len
         if window:
             span = min(span, window + 64)
         # about a thousand waves, one per SIMD of the chip, was the fastest at every batch size measured
@@ -171,7 +173,7 @@ class NativeBackend:
         M, K = x.shape
         N = w.shape[0]
         if x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
-            if M <= 16 or (M <= 64 and self.own_kernels_only):
+            if M <= self.few_rows or (M <= 64 and self.own_kernels_only):
                 return self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
                                   dtype_code(out), _stream())
             if out.dtype == torch.bfloat16 and bias is None and not self.own_kernels_only:
@@ -192,7 +194,7 @@ class NativeBackend:
         """silu(x Wg^T) * (x Wu^T) in one kernel, if this batch is one for the few-rows kernel; else False."""
         M, K = x.shape
         if (x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
-                and (M <= 16 or (M <= 64 and self.own_kernels_only))):
+                and (M <= self.few_rows or (M <= 64 and self.own_kernels_only))):
             self._call("nhv_gemm_skinny_glu_bf16", _ptr(x), _ptr(w), _ptr(out), M, out.shape[1], K, dtype_code(out),
                        _stream())
             return True

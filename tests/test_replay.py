@@ -174,6 +174,39 @@ def test_replay_at_the_family_head_size(model_folders, dtype, graphs):
             _check(got, want, tolerance_for(dtype, want), f"{dtype} head size 128, pages of {page}, {mode}")
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_steps_of_many_requests_replay_checked_graphs(model_folders, dtype):
+    """Steps of 17 to 64 single tokens: in bfloat16 their graphs hold the library's matrix products and are
+    checked when recorded (replayed three times between eager work, compared bit by bit). 40 requests decode
+    side by side, 15 of them end, the rest goes on: buckets of 64 and 32, every logit against the plain
+    implementation."""
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    folder = model_folders["D"]
+    cfg, w = plain.read_model_folder(folder)
+    requests = {f"r{i}": rc.random_tokens(cfg["vocab_size"], 30 + (i * 7) % 23 + (20 if i >= 15 else 0), 400 + i)
+                for i in range(40)}
+    prompt = 18
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:prompt], "want": [prompt - 1]}
+                                     for rid, toks in requests.items()], "end": []}]
+    fed = {rid: prompt for rid in requests}
+    while any(fed[rid] < len(toks) for rid, toks in requests.items()):
+        entries = [{"id": rid, "tokens": [toks[fed[rid]]], "want": [0]} for rid, toks in requests.items() if fed[rid] < len(toks)]
+        for e in entries:
+            fed[e["id"]] += 1
+        steps.append({"step": len(steps), "entries": entries,
+                      "end": [e["id"] for e in entries if fed[e["id"]] == len(requests[e["id"]])]})
+    sizes = {len(s["entries"]) for s in steps[1:]}
+    assert max(sizes) == 40 and any(16 < n <= 32 for n in sizes)
+    runner = ModelRunner(folder, dtype=dtype, page_size=64, num_pages=2 * len(requests) + 1, num_state_slots=40,
+                         use_graphs=True, max_model_len=128)
+    got = rc.run_in_process(runner, steps)
+    want = {rid: plain.logits(cfg, w, toks)[prompt - 1:] for rid, toks in requests.items()}
+    _check(got, want, tolerance_for(dtype, want), f"{dtype} decoding of 40 requests through graphs")
+    stats = runner.get_memory_stats()
+    assert {32, 64} <= set(stats["graphs_recorded"]) and stats["graphs_refused"] == [], stats
+
+
 def _trace_run(folder, dtype, steps, out_dir, max_tokens, extra=()):
     cmd = [sys.executable, os.path.join(REPO, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
            "--out", out_dir, "--max-tokens", str(max_tokens), *extra]
