@@ -86,6 +86,9 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
         self.max_model_len = min(max_model_len or self.max_position, self.max_position)
         self.max_graph_batch = max_graph_batch
+        # batch sizes that have a graph: a step is padded to the next one (powers of two and the sizes half way between)
+        sizes = sorted({b for p in range(8) for b in (1 << p, 3 << p >> 1) if b >= 1})
+        self.graph_buckets = [b for b in sizes if b < max_graph_batch] + [max_graph_batch]
         self._graphs: dict[int, dict | None] = {}     # None: the bucket's graph failed its check
 
     # ------------------------------------------------------------------ cache
@@ -359,9 +362,7 @@ class ModelRunner:
         entries and of each entry's ``want`` (None if nothing is wanted)."""
         if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)
                 and not self.state_pools):
-            bucket = 1
-            while bucket < len(entries):
-                bucket *= 2
+            bucket = next(b for b in self.graph_buckets if b >= len(entries))
             if self._graphs.get(bucket, ...) is not None:
                 return self._graph_step(entries, bucket)
         ctx, new_lens = self.build_context(entries)

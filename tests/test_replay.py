@@ -179,7 +179,7 @@ def test_replay_at_the_family_head_size(model_folders, dtype, graphs):
 def test_decoding_steps_of_many_requests_replay_checked_graphs(model_folders, dtype):
     """Steps of 17 to 64 single tokens: in bfloat16 their graphs hold the library's matrix products and are
     checked when recorded (replayed three times between eager work, compared bit by bit). 40 requests decode
-    side by side, 15 of them end, the rest goes on: buckets of 64 and 32, every logit against the plain
+    side by side, 15 of them end, the rest goes on: graphs of more than 16 rows, every logit against the plain
     implementation."""
     from nanohybrid_vlm_amd.engine.runner import ModelRunner
     folder = model_folders["D"]
@@ -204,7 +204,8 @@ def test_decoding_steps_of_many_requests_replay_checked_graphs(model_folders, dt
     want = {rid: plain.logits(cfg, w, toks)[prompt - 1:] for rid, toks in requests.items()}
     _check(got, want, tolerance_for(dtype, want), f"{dtype} decoding of 40 requests through graphs")
     stats = runner.get_memory_stats()
-    assert {32, 64} <= set(stats["graphs_recorded"]) and stats["graphs_refused"] == [], stats
+    recorded = stats["graphs_recorded"]
+    assert max(recorded) >= 40 and any(16 < b <= 32 for b in recorded) and stats["graphs_refused"] == [], stats
 
 
 def _trace_run(folder, dtype, steps, out_dir, max_tokens, extra=()):
