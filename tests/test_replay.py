@@ -208,6 +208,31 @@ def test_decoding_steps_of_many_requests_replay_checked_graphs(model_folders, dt
     assert max(recorded) >= 40 and any(16 < b <= 32 for b in recorded) and stats["graphs_refused"] == [], stats
 
 
+@pytest.mark.gpu
+def test_a_graph_that_fails_its_check_is_not_used(model_folders, capfd):
+    """The check of a graph with library calls in it is made to fail from the host: the step that recorded it
+    returns the eager result, later steps of that size run eagerly, and every logit is still right."""
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    folder = model_folders["D"]
+    cfg, w = plain.read_model_folder(folder)
+    requests = {f"r{i}": rc.random_tokens(cfg["vocab_size"], 24 + i % 3, 900 + i) for i in range(20)}
+    prompt = 18
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:prompt], "want": [prompt - 1]}
+                                     for rid, toks in requests.items()], "end": []}]
+    for t in range(prompt, 26):
+        entries = [{"id": rid, "tokens": [toks[t]], "want": [0]} for rid, toks in requests.items() if t < len(toks)]
+        steps.append({"step": len(steps), "entries": entries, "end": [e["id"] for e in entries if t == len(requests[e["id"]]) - 1]})
+    runner = ModelRunner(folder, dtype="bfloat16", page_size=64, num_pages=len(requests) + 1, num_state_slots=20,
+                         use_graphs=True, max_model_len=64)
+    runner.graph_check = lambda replayed, eager: False
+    got = rc.run_in_process(runner, steps)
+    want = {rid: plain.logits(cfg, w, toks)[prompt - 1:] for rid, toks in requests.items()}
+    _check(got, want, tolerance_for("bfloat16", want), "decoding of 20 requests with refused graphs")
+    stats = runner.get_memory_stats()
+    assert stats["graphs_refused"] == [24] and all(b <= 16 for b in stats["graphs_recorded"]), stats
+    assert "run eagerly" in capfd.readouterr().err
+
+
 def _trace_run(folder, dtype, steps, out_dir, max_tokens, extra=()):
     cmd = [sys.executable, os.path.join(REPO, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
            "--out", out_dir, "--max-tokens", str(max_tokens), *extra]
