@@ -21,7 +21,10 @@
 // doing the queries' norm and rotation and the cache write of the new key and value inside
 // this kernel instead of in one of their own: every split's wave then prepares the queries
 // again and waits for those loads before its first product, which gave back 4 of the 6
-// microseconds saved at 8 requests and lost time at 1 and at 64.)
+// microseconds saved at 8 requests and lost time at 1 and at 64. So were rounds of 64 keys for launches of one
+// wave per SIMD (5 % less time at 1 and 2 requests, more at 4 and above), and values loaded straight into LDS
+// (global_load_lds, read with ds_read_b64_tr_b16 as in the prompt kernel) with the next round's keys and values
+// asked for before this round is computed: 3 to 8 % less time for this kernel, 1 % of a decoding step.)
 #include "nhv_common.h"
 #include <math.h>
 
