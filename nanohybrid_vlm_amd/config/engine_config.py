@@ -55,6 +55,8 @@ class EngineConfig:
             raise ValueError("num_kvcache_blocks must be -1 or positive")
         if self.num_state_slots != -1 and self.num_state_slots <= 0:
             raise ValueError("num_state_slots must be -1 or positive")
+        if self.max_graph_batch <= 0:
+            raise ValueError("max_graph_batch must be positive")
 
     @classmethod
     def field_names(cls) -> set[str]:

@@ -87,7 +87,7 @@ class ModelRunner:
         self.max_model_len = min(max_model_len or self.max_position, self.max_position)
         self.max_graph_batch = max_graph_batch
         # batch sizes that have a graph: a step is padded to the next one (powers of two and the sizes half way between)
-        sizes = sorted({b for p in range(8) for b in (1 << p, 3 << p >> 1) if b >= 1})
+        sizes = sorted({b for p in range(24) for b in (1 << p, 3 << p >> 1) if b >= 1})
         self.graph_buckets = [b for b in sizes if b < max_graph_batch] + [max_graph_batch]
         self._graphs: dict[int, dict | None] = {}     # None: the bucket's graph failed its check
         self.graph_check = torch.equal                # (replay, eager) -> bool; a test replaces it to force a refusal

@@ -66,7 +66,7 @@ def test_engine_config_checks():
     assert EngineConfig(model="x", kvcache_block_size=4).kvcache_block_size == 4
     for bad in [dict(dtype="float16"), dict(scheduler_policy="fifo"), dict(max_prefill_wait_ms=-1),
                 dict(max_num_seqs=0), dict(gpu_memory_utilization=1.5), dict(kvcache_block_size=0),
-                dict(num_kvcache_blocks=0), dict(num_state_slots=-2)]:
+                dict(num_kvcache_blocks=0), dict(num_state_slots=-2), dict(max_graph_batch=0)]:
         with pytest.raises(ValueError):
             EngineConfig(model="x", **bad)
 

@@ -84,3 +84,12 @@ def test_bad_entries_are_refused(runner):
         runner._layout([StepEntry("c", [1] * 161, [])])
     runner.cache.check()
     assert np.asarray(runner.cache.block_table("c")).size == 0     # all or nothing
+
+
+def test_graph_buckets_are_powers_of_two_and_the_sizes_half_way_up_to_the_limit(emulated_kernels, model_folders):
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    for limit, want in [(64, [1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64]), (16, [1, 2, 3, 4, 6, 8, 12, 16]),
+                        (20, [1, 2, 3, 4, 6, 8, 12, 16, 20]), (1, [1])]:
+        runner = ModelRunner(model_folders["A"], dtype="float32", device="cpu", page_size=4, num_pages=8, num_state_slots=2,
+                             max_graph_batch=limit)
+        assert runner.graph_buckets == want
