@@ -39,7 +39,9 @@
 // It needs about 335 registers: with one wave per SIMD it reached 550 TFLOP/s where this kernel reaches 630 (8,192
 // tokens), held to two waves per SIMD it spills (250). With one wave per SIMD that loop ran at 1,280 TFLOP/s with
 // its matrix instructions alone, 860 with the LDS reads, 900 with the exponentials, 760 with both, and 500-550 with
-// the loads into LDS and the barrier of each tile.
+// the loads into LDS and the barrier of each tile. More waves do not help either: one row tile a wave, tiles of
+// 32 keys and four waves per SIMD (128 registers, 36 KB of LDS a block) reached 550 TFLOP/s, since every wave then
+// reads all keys and values from LDS for half as many rows.
 #include "nhv_common.h"
 #include <math.h>
 
