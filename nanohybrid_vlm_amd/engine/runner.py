@@ -91,6 +91,7 @@ class ModelRunner:
         self.graph_buckets = [b for b in sizes if b < max_graph_batch] + [max_graph_batch]
         self._graphs: dict[int, dict | None] = {}     # None: the bucket's graph failed its check
         self.graph_check = torch.equal                # (replay, eager) -> bool; a test replaces it to force a refusal
+        self.graphs_rerecorded = 0                    # graphs recorded again because the contexts had outgrown their layout
 
     # ------------------------------------------------------------------ cache
     def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens):
@@ -391,7 +392,12 @@ class ModelRunner:
         if meta["max_context_len"] > width * self.page_size:
             raise ValueError(f"a request of {meta['max_context_len']} tokens exceeds max_model_len {self.max_model_len}")
         g = self._graphs.get(bucket)
-        if g is None:
+        # a graph's kernels are laid out for the context lengths of the step that recorded it, g["planned"]; when the
+        # longest context is half as long again, or less than half of it, a new graph is recorded (the old one is dropped)
+        # (no graph is made for less than 256 keys: short contexts share one)
+        longest = max(256, meta["max_context_len"])
+        if g is None or not g["planned"] // 2 < longest <= g["planned"] + g["planned"] // 2:
+            self.graphs_rerecorded += g is not None
             g = self._capture(bucket, arrays, meta, width)
             self._graphs[bucket] = g if g["graph"] is not None else None
         if g["graph"] is not None:
@@ -424,9 +430,12 @@ class ModelRunner:
         ctx = self._context(dev, meta, all_rows, bucket, max_context_len=width * self.page_size)
         backend = ops.backend()
         with_library = bucket > getattr(backend, "few_rows", bucket) and self.dtype == torch.bfloat16
-        old = (getattr(backend, "own_kernels_only", False), getattr(backend, "recording_graph", False))
+        old = (getattr(backend, "own_kernels_only", False), getattr(backend, "planned_context", 0))
         backend.own_kernels_only = not with_library
-        backend.recording_graph = True                      # lengths are only bounded: kernels plan for the bound
+        # the graph's launches are fixed: kernels that split the keys plan for this step's longest context (replays
+        # with other lengths stay right: the block tables and the splits' results are made for max_model_len)
+        planned = max(256, meta["max_context_len"])
+        backend.planned_context = planned
         try:
             # warm-up; it writes the same cache slots as every replay will
             eager = self.model.logits(self.model.forward(ctx)).clone()
@@ -442,12 +451,12 @@ class ModelRunner:
                     if not self.graph_check(logits, eager):
                         print(f"[nanohybrid_vlm_amd] the graph for {bucket} requests differs from the eager step when "
                               "replayed; steps of this size run eagerly", file=sys.stderr, flush=True)
-                        return {"graph": None, "index": index, "logits": eager, "ctx": ctx}
+                        return {"graph": None, "index": index, "logits": eager, "ctx": ctx, "planned": planned}
                     self.model.logits(self.model.forward(ctx))      # eager work between the replays
                     torch.cuda.synchronize()
         finally:
-            backend.own_kernels_only, backend.recording_graph = old
-        return {"graph": graph, "index": index, "logits": logits, "ctx": ctx}
+            backend.own_kernels_only, backend.planned_context = old
+        return {"graph": graph, "index": index, "logits": logits, "ctx": ctx, "planned": planned}
 
     def get_memory_stats(self) -> dict:
         """Bytes of weights, cache and state pools, pages per group, and the allocator's and the device's view
@@ -470,6 +479,7 @@ class ModelRunner:
                              "shared_tokens": self.cache.num_shared_tokens},
             "graphs_recorded": sorted(b for b, g in self._graphs.items() if g is not None),
             "graphs_refused": sorted(b for b, g in self._graphs.items() if g is None),
+            "graphs_rerecorded": self.graphs_rerecorded,
         }
         if self.device.type == "cuda":
             free, total = torch.cuda.mem_get_info(self.device)

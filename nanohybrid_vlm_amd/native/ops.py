@@ -80,7 +80,7 @@ class NativeBackend:
     device_type = "cuda"
     few_rows = 16                 # up to this many rows the own matrix kernels are the faster ones
     own_kernels_only = False      # True: no library call (matrix products of up to 64 rows take the own kernels)
-    recording_graph = False       # True while a HIP graph is recorded: lengths are bounds, not the step's own
+    planned_context = 0           # > 0 while a HIP graph is recorded: the lengths to plan for (the batch's own are bounds)
 
     def __init__(self):
         if not torch.cuda.is_available():
@@ -151,8 +151,8 @@ class NativeBackend:
         """Single tokens in bfloat16: keys split over waves, then merged."""
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
-        # inside a graph the lengths are only bounded (by max_model_len): plan for half the bound
-        span = batch.max_context_len // 2 if self.recording_graph else batch.max_context_len
+        # inside a graph the lengths are only bounded (by max_model_len): the recorder says what to plan for
+        span = min(self.planned_context, batch.max_context_len) if self.planned_context else batch.max_context_len
         if window:
             span = min(span, window + 64)
         # about a thousand waves, one per SIMD of the chip, was the fastest at every batch size measured

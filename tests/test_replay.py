@@ -151,6 +151,9 @@ def test_long_decoding_and_first_tokens(model_folders, dtype, graphs):
                          max_model_len=512)
     got = rc.run_in_process(runner, steps)
     _check(got, {"a": plain.logits(cfg, w, a), "b": plain.logits(cfg, w, b)}, TOLERANCE[dtype], f"{dtype} long decoding")
+    if graphs:
+        # a graph's kernels are laid out for the contexts of the step that recorded it: past 384 keys it is recorded again
+        assert runner.get_memory_stats()["graphs_rerecorded"] >= 1
 
 
 @pytest.mark.gpu
