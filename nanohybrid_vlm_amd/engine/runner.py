@@ -77,12 +77,12 @@ class ModelRunner:
         # request no longer owns shows up in its logits
         self.poison_freed_pages = poison_freed_pages
         # decode-only steps replay a HIP graph per batch-size bucket (the reference captures CUDA graphs for
-        # the same batch sizes, nanovllm/engine/model_runner.py:2559-2594). Up to 16 requests the graph holds
-        # own kernels only. Larger buckets hold the library's matrix products too (measured faster than the own
-        # kernel from 17 rows on), and a step of 17 to 48 requests is bound by its launches when run eagerly
-        # (8.3 ms at every size). A graph with a library call in it is checked when it is recorded: replayed
-        # three times, with eager work and waits between, and compared bit by bit with the eager result;
-        # a bucket whose graph fails runs eagerly from then on.
+        # the same batch sizes, nanovllm/engine/model_runner.py:2559-2594). In bfloat16 a graph may hold the
+        # library's matrix products beside the own kernels: from 17 rows on always (measured faster than the own
+        # kernel there), for fewer rows where a measurement of the shape says so. Run eagerly, a step of 17 to 48
+        # requests is bound by its launches (8.3 ms at every size). A graph with a library call in it is checked
+        # when it is recorded: replayed three times, with eager work and waits between, and compared bit by bit
+        # with the eager result; a bucket whose graph fails runs eagerly from then on.
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
         self.max_model_len = min(max_model_len or self.max_position, self.max_position)
         self.max_graph_batch = max_graph_batch
@@ -429,9 +429,11 @@ class ModelRunner:
         all_rows = torch.arange(bucket, dtype=torch.int32, device=self.device)
         ctx = self._context(dev, meta, all_rows, bucket, max_context_len=width * self.page_size)
         backend = ops.backend()
-        with_library = bucket > getattr(backend, "few_rows", bucket) and self.dtype == torch.bfloat16
-        old = (getattr(backend, "own_kernels_only", False), getattr(backend, "planned_context", 0))
-        backend.own_kernels_only = not with_library
+        with_library = self.dtype == torch.bfloat16           # (the float32 path has kernels of its own throughout)
+        old = (getattr(backend, "own_kernels_only", False), getattr(backend, "planned_context", 0),
+               getattr(backend, "measure_linears", False))
+        backend.own_kernels_only = False
+        backend.measure_linears = True                        # few-rows products of new shapes are timed both ways, once
         # the graph's launches are fixed: kernels that split the keys plan for this step's longest context (replays
         # with other lengths stay right: the block tables and the splits' results are made for max_model_len)
         planned = max(256, meta["max_context_len"])
@@ -455,7 +457,7 @@ class ModelRunner:
                     self.model.logits(self.model.forward(ctx))      # eager work between the replays
                     torch.cuda.synchronize()
         finally:
-            backend.own_kernels_only, backend.planned_context = old
+            backend.own_kernels_only, backend.planned_context, backend.measure_linears = old
         return {"graph": graph, "index": index, "logits": logits, "ctx": ctx, "planned": planned}
 
     def get_memory_stats(self) -> dict:

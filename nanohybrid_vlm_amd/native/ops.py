@@ -81,6 +81,7 @@ class NativeBackend:
     few_rows = 16                 # up to this many rows the own matrix kernels are the faster ones
     own_kernels_only = False      # True: no library call (matrix products of up to 64 rows take the own kernels)
     planned_context = 0           # > 0 while a HIP graph is recorded: the lengths to plan for (the batch's own are bounds)
+    measure_linears = False       # True: a few-rows product of a shape not seen before is timed both ways (see linear)
 
     def __init__(self):
         if not torch.cuda.is_available():
@@ -88,6 +89,7 @@ class NativeBackend:
         self.lib = library.load_library("nhv_core", CORE_SOURCES)
         self.lib.nhv_last_error.restype = ctypes.c_char_p
         self._attention_libs: dict[int, ctypes.CDLL] = {}
+        self.library_is_faster: dict[tuple[int, int, int], bool] = {}     # (M, N, K) of few-rows products -> measured
 
     def _call(self, fn_name: str, *args, lib=None) -> None:
         lib = lib or self.lib
@@ -169,10 +171,48 @@ class NativeBackend:
                    block_tables.shape[1], T, Hq, Hkv, page_size, ctypes.c_float(scale), window, split_len, n_splits,
                    _stream(), lib=self.attention_lib(D))
 
+    def _few_rows_by_library(self, x, w, out) -> bool:
+        """Whether this product of up to ``few_rows`` rows goes to the library. The own kernel is the rule; which
+        of the two is faster depends on the shape in ways no rule here captures (at 8 rows the library takes 21
+        against 25 us for a 4096 x 12288 matrix and 112 against 50 us for a 5120 x 17408 one), so while
+        ``measure_linears`` is set (the run before a graph is recorded) a shape not seen before is timed both
+        ways, and the answer is kept for the life of the process."""
+        key = (x.shape[0], w.shape[0], w.shape[1])
+        known = self.library_is_faster.get(key)
+        if known is not None or not self.measure_linears or torch.cuda.is_current_stream_capturing():
+            return bool(known)
+        M, K = x.shape
+
+        def own():
+            self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), None, _ptr(out), M, w.shape[0], K, dtype_code(out), _stream())
+
+        def library():
+            torch.mm(x, w.t(), out=out)
+
+        best = {}
+        for name, run in (("own", own), ("library", library)):
+            run()                                            # loads what the call needs
+            times = []
+            for _ in range(3):
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                run()
+                run()
+                end.record()
+                end.synchronize()
+                times.append(start.elapsed_time(end))
+            best[name] = min(times)
+        self.library_is_faster[key] = best["library"] < 0.95 * best["own"]
+        return self.library_is_faster[key]
+
     def linear(self, x, w, bias, out):
         M, K = x.shape
         N = w.shape[0]
         if x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
+            if M <= self.few_rows and out.dtype == torch.bfloat16 and bias is None and not self.own_kernels_only \
+                    and self._few_rows_by_library(x, w, out):
+                torch.mm(x, w.t(), out=out)
+                return None
             if M <= self.few_rows or (M <= 64 and self.own_kernels_only):
                 return self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
                                   dtype_code(out), _stream())

@@ -232,7 +232,7 @@ def test_a_graph_that_fails_its_check_is_not_used(model_folders, capfd):
     want = {rid: plain.logits(cfg, w, toks)[prompt - 1:] for rid, toks in requests.items()}
     _check(got, want, tolerance_for("bfloat16", want), "decoding of 20 requests with refused graphs")
     stats = runner.get_memory_stats()
-    assert stats["graphs_refused"] == [24] and all(b <= 16 for b in stats["graphs_recorded"]), stats
+    assert 24 in stats["graphs_refused"] and stats["graphs_recorded"] == [], stats
     assert "run eagerly" in capfd.readouterr().err
 
 
