@@ -89,7 +89,7 @@ class NativeBackend:
         self.lib = library.load_library("nhv_core", CORE_SOURCES)
         self.lib.nhv_last_error.restype = ctypes.c_char_p
         self._attention_libs: dict[int, ctypes.CDLL] = {}
-        self.library_is_faster: dict[tuple[int, int, int], bool] = {}     # (M, N, K) of few-rows products -> measured
+        self.library_is_faster: dict[tuple, bool] = {}     # (M, N, K, gated) of few-rows products -> measured
 
     def _call(self, fn_name: str, *args, lib=None) -> None:
         lib = lib or self.lib
@@ -171,26 +171,11 @@ class NativeBackend:
                    block_tables.shape[1], T, Hq, Hkv, page_size, ctypes.c_float(scale), window, split_len, n_splits,
                    _stream(), lib=self.attention_lib(D))
 
-    def _few_rows_by_library(self, x, w, out) -> bool:
-        """Whether this product of up to ``few_rows`` rows goes to the library. The own kernel is the rule; which
-        of the two is faster depends on the shape in ways no rule here captures (at 8 rows the library takes 21
-        against 25 us for a 4096 x 12288 matrix and 112 against 50 us for a 5120 x 17408 one), so while
-        ``measure_linears`` is set (the run before a graph is recorded) a shape not seen before is timed both
-        ways, and the answer is kept for the life of the process."""
-        key = (x.shape[0], w.shape[0], w.shape[1])
-        known = self.library_is_faster.get(key)
-        if known is not None or not self.measure_linears or torch.cuda.is_current_stream_capturing():
-            return bool(known)
-        M, K = x.shape
-
-        def own():
-            self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), None, _ptr(out), M, w.shape[0], K, dtype_code(out), _stream())
-
-        def library():
-            torch.mm(x, w.t(), out=out)
-
-        best = {}
-        for name, run in (("own", own), ("library", library)):
+    @staticmethod
+    def _faster(first, second) -> bool:
+        """Whether ``second()`` takes less than 0.95 of the time of ``first()`` on the GPU (best of three pairs)."""
+        best = []
+        for run in (first, second):
             run()                                            # loads what the call needs
             times = []
             for _ in range(3):
@@ -201,8 +186,40 @@ class NativeBackend:
                 end.record()
                 end.synchronize()
                 times.append(start.elapsed_time(end))
-            best[name] = min(times)
-        self.library_is_faster[key] = best["library"] < 0.95 * best["own"]
+            best.append(min(times))
+        return best[1] < 0.95 * best[0]
+
+    def _few_rows_by_library(self, x, w, out, gated: bool = False) -> bool:
+        """Whether this product of up to ``few_rows`` rows goes to the library (``gated``: followed by the
+        SiLU-and-multiply kernel, instead of the own kernel that does both). The own kernel is the rule; which
+        of the two is faster depends on the shape in ways no rule here captures (at 8 rows the library takes 21
+        against 25 us for a 4096 x 12288 matrix and 112 against 50 us for a 5120 x 17408 one), so while
+        ``measure_linears`` is set (the run before a graph is recorded) a shape not seen before is timed both
+        ways, and the answer is kept for the life of the process."""
+        M, K = x.shape
+        N = w.shape[0]
+        key = (M, N, K, gated)
+        known = self.library_is_faster.get(key)
+        if known is not None or not self.measure_linears or torch.cuda.is_current_stream_capturing():
+            return bool(known)
+        if gated:
+            packed = torch.empty((M, N), dtype=x.dtype, device=x.device)
+
+            def own():
+                self._call("nhv_gemm_skinny_glu_bf16", _ptr(x), _ptr(w), _ptr(out), M, N // 2, K, dtype_code(out), _stream())
+
+            def library():
+                torch.mm(x, w.t(), out=packed)
+                self.silu_mul(packed, out)
+        else:
+            def own():
+                self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), None, _ptr(out), M, N, K, dtype_code(out), _stream())
+
+            def library():
+                torch.mm(x, w.t(), out=out)
+        self.library_is_faster[key] = self._faster(own, library)
+        if gated and self.library_is_faster[key]:
+            self.library_is_faster[(M, N, K, False)] = True  # the packed product that follows a refusal of gated_linear
         return self.library_is_faster[key]
 
     def linear(self, x, w, bias, out):
@@ -235,6 +252,8 @@ class NativeBackend:
         M, K = x.shape
         if (x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
                 and (M <= self.few_rows or (M <= 64 and self.own_kernels_only))):
+            if M <= self.few_rows and not self.own_kernels_only and self._few_rows_by_library(x, w, out, gated=True):
+                return False                                 # the library's product, then silu_mul
             self._call("nhv_gemm_skinny_glu_bf16", _ptr(x), _ptr(w), _ptr(out), M, out.shape[1], K, dtype_code(out),
                        _stream())
             return True
