@@ -40,23 +40,34 @@ def _ptr(t: torch.Tensor | None):
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """torch's current stream of the current device, as the kernels' launch argument (asked for before every
+    kernel: the direct call takes a tenth of the time of building a ``torch.cuda.Stream`` object)."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def _need(cond: bool, msg: str) -> None:
+def _need(cond: bool, msg) -> None:
+    """``msg``: the message, or a function that makes it (the checks run before every kernel: a message that
+    has to be formatted is only formatted when the check fails)."""
     if not cond:
-        raise KernelError(msg)
+        raise KernelError(msg() if callable(msg) else msg)
 
 
 def _dense(t: torch.Tensor, name: str, shape: tuple | None = None, dtype=None) -> None:
     want = backend().device_type
-    _need(t.device.type == want, f"{name}: must live on a '{want}' device, is on {t.device}")
-    _need(t.is_contiguous(), f"{name}: must be contiguous")
-    if shape is not None:
-        _need(tuple(t.shape) == tuple(shape), f"{name}: shape {tuple(t.shape)} but {tuple(shape)} is needed")
-    if dtype is not None:
-        _need(t.dtype == dtype, f"{name}: element type {t.dtype} but {dtype} is needed")
+    if t.device.type != want:
+        raise KernelError(f"{name}: must live on a '{want}' device, is on {t.device}")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: must be contiguous")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name}: shape {tuple(t.shape)} but {tuple(shape)} is needed")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: element type {t.dtype} but {dtype} is needed")
 
 
 @dataclass
@@ -351,7 +362,7 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, residual: torch.Tensor
     _dense(x, "rmsnorm: x")
     _dense(w, "rmsnorm: weight", (x.shape[1],))
     _need(w.dtype == x.dtype or w.dtype == torch.float32,
-          f"rmsnorm: weight of {w.dtype} with activations of {x.dtype}")
+          lambda: f"rmsnorm: weight of {w.dtype} with activations of {x.dtype}")
     dtype_code(x)
     y = torch.empty_like(x)
     if start_residual:
@@ -362,7 +373,7 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, residual: torch.Tensor
     if residual is not None:
         _dense(residual, "rmsnorm: residual", tuple(x.shape))
         _need(residual.dtype == x.dtype or residual.dtype == torch.float32,
-              f"rmsnorm: residual of {residual.dtype} with rows of {x.dtype}")
+              lambda: f"rmsnorm: residual of {residual.dtype} with rows of {x.dtype}")
         backend().rmsnorm(x, residual, 1, w, y, float(eps))
         return y
     backend().rmsnorm(x, None, 0, w, y, float(eps))
@@ -401,7 +412,7 @@ def qk_rope_write(qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, positions, slot_m
     for name, w in (("q_norm", q_norm_w), ("k_norm", k_norm_w)):
         if w is not None:
             _dense(w, f"qk_rope_write: {name} weight", (head_dim,))
-            _need(w.dtype == qkv.dtype or w.dtype == torch.float32, f"qk_rope_write: {name} weight of {w.dtype}")
+            _need(w.dtype == qkv.dtype or w.dtype == torch.float32, lambda: f"qk_rope_write: {name} weight of {w.dtype}")
     _need((q_norm_w is None) == (k_norm_w is None), "qk_rope_write: q and k norm weights come together")
     if q_norm_w is not None:
         _need(q_norm_w.dtype == k_norm_w.dtype, "qk_rope_write: q and k norm weights differ in element type")
@@ -410,12 +421,12 @@ def qk_rope_write(qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, positions, slot_m
         _need(cos_sin.dim() == 2, "qk_rope_write: rotation table must be [positions, rotary size]")
         _dense(cos_sin, "qk_rope_write: rotation table", dtype=torch.float32)
         rot = cos_sin.shape[1]
-        _need(rot % 2 == 0 and rot <= head_dim, f"qk_rope_write: rotary size {rot} with head size {head_dim}")
+        _need(rot % 2 == 0 and rot <= head_dim, lambda: f"qk_rope_write: rotary size {rot} with head size {head_dim}")
     _dense(positions, "qk_rope_write: positions", (T,), torch.int32)
     if write_kv:
         _dense(slot_mapping, "qk_rope_write: slot_mapping", (T,), torch.int32)
         _need(k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (num_kv_heads, head_dim),
-              f"qk_rope_write: cache shape {tuple(k_cache.shape)} does not fit {num_kv_heads} heads of {head_dim}")
+              lambda: f"qk_rope_write: cache shape {tuple(k_cache.shape)} does not fit {num_kv_heads} heads of {head_dim}")
         _dense(k_cache, "qk_rope_write: k_cache", dtype=qkv.dtype)
         _dense(v_cache, "qk_rope_write: v_cache", tuple(k_cache.shape), qkv.dtype)
     q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
@@ -431,20 +442,20 @@ def paged_attention(q, k_cache, v_cache, batch: AttentionBatch, block_tables, sc
     T, Hq, D = q.shape
     _dense(q, "attention: q")
     dtype_code(q)
-    _need(k_cache.dim() == 4 and k_cache.shape[3] == D, f"attention: cache shape {tuple(k_cache.shape)} with head size {D}")
+    _need(k_cache.dim() == 4 and k_cache.shape[3] == D, lambda: f"attention: cache shape {tuple(k_cache.shape)} with head size {D}")
     _dense(k_cache, "attention: k_cache", dtype=q.dtype)
     _dense(v_cache, "attention: v_cache", tuple(k_cache.shape), q.dtype)
     Hkv = k_cache.shape[2]
-    _need(Hq % Hkv == 0, f"attention: {Hq} query heads are not a multiple of {Hkv} key heads")
-    _need(T == batch.num_tokens, f"attention: {T} tokens but the batch has {batch.num_tokens}")
+    _need(Hq % Hkv == 0, lambda: f"attention: {Hq} query heads are not a multiple of {Hkv} key heads")
+    _need(T == batch.num_tokens, lambda: f"attention: {T} tokens but the batch has {batch.num_tokens}")
     _dense(batch.token_req, "attention: token_req", (T,), torch.int32)
     _dense(batch.positions, "attention: positions", (T,), torch.int32)
     _need(block_tables.dim() == 2 and block_tables.shape[0] == batch.num_requests,
-          f"attention: block tables {tuple(block_tables.shape)} for {batch.num_requests} requests")
+          lambda: f"attention: block tables {tuple(block_tables.shape)} for {batch.num_requests} requests")
     _dense(block_tables, "attention: block_tables", dtype=torch.int32)
     page_size = k_cache.shape[1]
     _need(block_tables.shape[1] * page_size >= batch.max_context_len,
-          f"attention: block tables of {block_tables.shape[1]} pages of {page_size} are too short for "
+          lambda: f"attention: block tables of {block_tables.shape[1]} pages of {page_size} are too short for "
           f"{batch.max_context_len} keys")
     out = torch.empty_like(q)
     backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), int(window or 0))
@@ -455,14 +466,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, o
     """x[M, K] . w[N, K]^T (+ bias), accumulated in float. ``out_dtype`` may be
     float32 for bfloat16 inputs (the logits)."""
     _need(x.dim() == 2 and w.dim() == 2, "linear: x must be [rows, in] and w [out, in]")
-    _need(x.shape[1] == w.shape[1], f"linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
+    _need(x.shape[1] == w.shape[1], lambda: f"linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
     _dense(x, "linear: x")
     _dense(w, "linear: w", dtype=x.dtype)
     dtype_code(x)
     if bias is not None:
         _dense(bias, "linear: bias", (w.shape[0],), x.dtype)
     out_dtype = out_dtype or x.dtype
-    _need(out_dtype == x.dtype or out_dtype == torch.float32, f"linear: output of {out_dtype} from {x.dtype}")
+    _need(out_dtype == x.dtype or out_dtype == torch.float32, lambda: f"linear: output of {out_dtype} from {x.dtype}")
     out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
     backend().linear(x, w, bias, out)
     return out
@@ -472,7 +483,7 @@ def gated_linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """silu(x . w[:I]^T) * (x . w[I:]^T) for a packed gate | up matrix w[2 I, K]: fused into one kernel for
     few rows, else the matrix product followed by ``silu_mul``."""
     _need(x.dim() == 2 and w.dim() == 2 and w.shape[0] % 2 == 0, "gated_linear: x must be [rows, in] and w [2 * out, in]")
-    _need(x.shape[1] == w.shape[1], f"gated_linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
+    _need(x.shape[1] == w.shape[1], lambda: f"gated_linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
     _dense(x, "gated_linear: x")
     _dense(w, "gated_linear: w", dtype=x.dtype)
     dtype_code(x)
