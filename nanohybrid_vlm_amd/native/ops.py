@@ -184,16 +184,16 @@ class NativeBackend:
 
     @staticmethod
     def _faster(first, second) -> bool:
-        """Whether ``second()`` takes less than 0.95 of the time of ``first()`` on the GPU (best of three pairs)."""
+        """Whether ``second()`` takes less than 0.95 of the time of ``first()`` on the GPU (best of five runs of four)."""
         best = []
         for run in (first, second):
             run()                                            # loads what the call needs
             times = []
-            for _ in range(3):
+            for _ in range(5):
                 start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 start.record()
-                run()
-                run()
+                for _ in range(4):
+                    run()
                 end.record()
                 end.synchronize()
                 times.append(start.elapsed_time(end))
