@@ -442,3 +442,36 @@ def test_refusals(ops):
         ops.rmsnorm(rnd(4, 128)[:, ::2], rnd(64), 1e-6)
     with pytest.raises(KernelError, match="device"):
         ops.rmsnorm(torch.zeros(2, 8), torch.ones(8), 1e-6)
+
+
+def test_few_rows_products_are_given_to_the_faster_of_own_kernel_and_library(ops):
+    """While ``measure_linears`` is set a shape not seen before is timed both ways and the answer kept; whichever
+    way a product goes, it is the same product."""
+    backend = ops.backend()
+    M, N, K = 8, 512, 1024
+    x = rnd(M, K, dtype=torch.bfloat16, seed=51)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=52, scale=K ** -0.5)
+    w2 = rnd(2 * N, K, dtype=torch.bfloat16, seed=53, scale=K ** -0.5)
+    ref = x.double() @ w.double().T
+    g, u = x.double() @ w2[:N].double().T, x.double() @ w2[N:].double().T
+    keys = [(M, N, K, False), (M, 2 * N, K, True)]
+    saved = {k: backend.library_is_faster.pop(k, None) for k in keys + [(M, 2 * N, K, False)]}
+    try:
+        assert ops.linear(x, w) is not None and keys[0] not in backend.library_is_faster      # not measured unasked
+        backend.measure_linears = True
+        try:
+            ops.linear(x, w)
+            ops.gated_linear(x, w2)
+        finally:
+            backend.measure_linears = False
+        assert all(isinstance(backend.library_is_faster[k], bool) for k in keys)
+        for by_library in (False, True):
+            for k in keys + [(M, 2 * N, K, False)]:
+                backend.library_is_faster[k] = by_library
+            torch.testing.assert_close(ops.linear(x, w).double(), ref, **tol(torch.bfloat16))
+            torch.testing.assert_close(ops.gated_linear(x, w2).double(), g * torch.sigmoid(g) * u, **tol(torch.bfloat16))
+    finally:
+        for k, v in saved.items():
+            backend.library_is_faster.pop(k, None)
+            if v is not None:
+                backend.library_is_faster[k] = v
