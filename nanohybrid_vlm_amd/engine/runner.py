@@ -458,6 +458,8 @@ class ModelRunner:
                     torch.cuda.synchronize()
         finally:
             backend.own_kernels_only, backend.planned_context, backend.measure_linears = old
+            if hasattr(backend, "end_measurements"):
+                backend.end_measurements()
         return {"graph": graph, "index": index, "logits": logits, "ctx": ctx, "planned": planned}
 
     def get_memory_stats(self) -> dict:

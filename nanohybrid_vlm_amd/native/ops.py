@@ -191,7 +191,10 @@ class NativeBackend:
         step a weight comes from memory, and a weight left in a cache by the run before would be measured 15 to
         20 % too fast, by an amount that differs between the two."""
         if self._sweep is None:
-            self._sweep = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+            try:
+                self._sweep = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+            except torch.OutOfMemoryError:
+                return False                                 # no room to measure: the own kernel, as the rule says
         best = []
         for run in (first, second):
             run()                                            # loads what the call needs
@@ -242,6 +245,10 @@ class NativeBackend:
         if gated and self.library_is_faster[key]:
             self.library_is_faster[(M, N, K, False)] = True  # the packed product that follows a refusal of gated_linear
         return self.library_is_faster[key]
+
+    def end_measurements(self) -> None:
+        """Gives the scratch memory of the measurements back (what was measured stays known)."""
+        self._sweep = None
 
     def linear(self, x, w, bias, out):
         M, K = x.shape
