@@ -14,7 +14,9 @@
 // then cross from L2 to a compute unit once per call instead of once per tile: 5 to 25 % less time at
 // every size measured, most where N is large (the head: 266 to 221 us at 8 rows). Where x does not
 // fit at once and w has at most 256 tiles, a third kernel gives every block one tile and takes x through
-// LDS in pieces (the 8B down projection from 7 rows on: 2 to 6 % less time, 12 % with 2,048 outputs).
+// LDS in pieces (the 8B down projection from 7 rows on: 2 to 6 % less time, 12 % with 2,048 outputs). With more
+// tiles than that, and x fitting in two pieces, a fourth kernel walks over all of a block's tiles once for each
+// piece and keeps the tiles' sums in LDS between the two (16 rows of 5,120 columns: 13 % less time for gate_up).
 //
 // How many tiles a block takes, how many waves share K and how many loads a wave keeps in flight is
 // chosen per call from M, N and K (plan() below): blocks that spread evenly over the compute units
@@ -311,6 +313,113 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const b
   }
 }
 
+// Where all of x is too much for LDS and a block has several tiles: x comes in `npasses` pieces of `pass_steps`
+// steps of 32 columns; for every piece the block walks over all of its tiles, and a tile's sums over the pieces so
+// far wait in LDS (part_s, 1 KB a tile and matrix) for the next piece. The weights are still read once. The
+// wave that adds up a tile's sums is the same in every pass, so what it left in part_s it finds again itself.
+template <int WAVES, int UNROLL, bool GLU, typename TOut>
+__global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_passes_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                           const bf16_t* __restrict__ bias, TOut* __restrict__ y,
+                                                                           int M, int N, int K, int tiles, int npasses,
+                                                                           int pass_steps, int steps_per_wave, int tiles_per_block) {
+  constexpr int NA = GLU ? 2 : 1;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  float(*red)[NA][4][64] = reinterpret_cast<float(*)[NA][4][64]>(lds_raw);      // [2 WAVES][NA][4][64]
+  float(*part_s)[NA][4][64] = red + 2 * WAVES;                                   // [tiles_per_block][NA][4][64]
+  bf16_t* x_s = reinterpret_cast<bf16_t*>(lds_raw + (size_t)(2 * WAVES + tiles_per_block) * NA * 4 * 64 * sizeof(float));
+  const int pitch = min(K, pass_steps * 32) + 8;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int ksteps = (K + 31) / 32;
+  const bool m_ok = col < M;
+  const bf16_t* xrow_s = x_s + (m_ok ? col : 0) * pitch;
+  int parity = 0;
+  for (int p = 0; p < npasses; ++p) {
+    const int c0 = p * pass_steps, c_end = min(c0 + pass_steps, ksteps);
+    // this piece of x into LDS: a wave's load brings 64 consecutive 16-byte pieces of one row
+    if (p > 0) __syncthreads();                          // the piece before has been read by every wave
+    {
+      const int col0 = c0 * 32;
+      const int pieces_per_row = (min(K, c_end * 32) - col0) / 8;
+      const int loads_per_row = (pieces_per_row + 63) / 64;
+      for (int job = wave; job < M * loads_per_row; job += WAVES) {
+        const int m = job / loads_per_row, part = job % loads_per_row;
+        const int piece = part * 64 + lane;
+        if (piece < pieces_per_row)
+          __builtin_amdgcn_global_load_lds((global_ptr)(x + (size_t)m * K + col0 + piece * 8),
+                                           (lds_ptr)(x_s + m * pitch + part * 512), 16, 0, 0);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
+    const int first = c0 + wave * steps_per_wave;
+    const int last = min(first + steps_per_wave, c_end);
+    int ti = 0, turn = 0;
+    for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x, ++ti, parity ^= 1, turn = turn + 1 == WAVES ? 0 : turn + 1) {
+      const int n0 = tile * 16;
+      const bool n_ok = n0 + col < N;
+      const bf16_t* wrow[NA];
+#pragma unroll
+      for (int na = 0; na < NA; ++na) wrow[na] = w + ((size_t)na * N + (n_ok ? n0 + col : 0)) * K;
+      floatx4 acc[NA];
+#pragma unroll
+      for (int na = 0; na < NA; ++na) acc[na] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int s0 = first; s0 < last; s0 += UNROLL) {
+        bf16x8 a[UNROLL][NA];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const int k = (s0 + u) * 32 + grp * 8;
+          const bool k_ok = (s0 + u < last) && k < K;
+#pragma unroll
+          for (int na = 0; na < NA; ++na) a[u][na] = (n_ok && k_ok) ? load8(wrow[na] + k) : zero8();
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const int k = (s0 + u) * 32 + grp * 8;
+          const bool k_ok = (s0 + u < last) && k < K;
+          const bf16x8 b = (m_ok && k_ok) ? *reinterpret_cast<const bf16x8*>(xrow_s + (k - c0 * 32)) : zero8();
+#pragma unroll
+          for (int na = 0; na < NA; ++na) acc[na] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][na], b, acc[na], 0, 0, 0);
+        }
+      }
+      float(*my_red)[NA][4][64] = red + parity * WAVES;
+#pragma unroll
+      for (int na = 0; na < NA; ++na)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) my_red[wave][na][j][lane] = acc[na][j];
+      __syncthreads();                        // the other buffer is the one written for the next tile
+      if (wave != turn) continue;
+      float v[NA][4];
+#pragma unroll
+      for (int na = 0; na < NA; ++na)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float sum = p > 0 ? part_s[ti][na][j][lane] : 0.f;
+#pragma unroll
+          for (int wv = 0; wv < WAVES; ++wv) sum += my_red[wv][na][j][lane];
+          v[na][j] = sum;
+        }
+      if (p + 1 < npasses) {
+#pragma unroll
+        for (int na = 0; na < NA; ++na)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) part_s[ti][na][j][lane] = v[na][j];
+        continue;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + grp * 4 + j;
+        if (col < M && n < N) {
+          float r = v[0][j];
+          if (bias) r += (float)bias[n];
+          if (GLU) r = r / (1.0f + expf(-r)) * v[NA - 1][j];
+          y[(size_t)col * N + n] = (TOut)r;
+        }
+      }
+    }
+  }
+}
+
 constexpr size_t LDS_BYTES = 160 * 1024;
 
 // The resident kernel's shape: waves, loads in flight and blocks per compute unit, from the best variants measured
@@ -390,6 +499,43 @@ static int launch_resident(const ResidentPlan& p, hipStream_t s, const void* x, 
   return 0;
 }
 
+// The shape of the kernel that takes x in pieces and walks over all of a block's tiles for every piece: one
+// block a compute unit; waves == 0 when it does not fit.
+struct PassesPlan {
+  int waves, unroll, npasses, pass_steps, tiles_per_block, grid;
+  size_t lds;
+};
+static PassesPlan passes_plan(bool glu, int M, int N, int K) {
+  const int tiles = (N + 15) / 16, ksteps = (K + 31) / 32;
+  const int grid = tiles < 256 ? tiles : 256;
+  const int tpb = (tiles + grid - 1) / grid;
+  int waves, unroll;
+  if (glu) waves = M <= 12 ? 8 : 4, unroll = M <= 12 ? 2 : 8;
+  else waves = M >= 13 ? 8 : 16, unroll = M >= 13 ? 8 : 2;
+  const int na = glu ? 2 : 1;
+  for (int npasses = 2; npasses <= 8; ++npasses) {
+    const int pass_steps = 2 * waves * ((ksteps + 2 * waves * npasses - 1) / (2 * waves * npasses));   // every wave whole lines
+    const int columns = pass_steps * 32 < K ? pass_steps * 32 : K;
+    const size_t lds = (size_t)(2 * waves + tpb) * na * 4 * 64 * sizeof(float) + (size_t)M * (columns + 8) * 2;
+    if (lds <= LDS_BYTES) return {waves, unroll, (ksteps + pass_steps - 1) / pass_steps, pass_steps, tpb, grid, lds};
+  }
+  return {0, 0, 0, 0, 0, 0, 0};
+}
+
+template <int WAVES, int UNROLL, bool GLU, typename TOut>
+static int launch_passes(const PassesPlan& p, hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M, int N,
+                         int K) {
+  auto kernel = gemm_fewrows_passes_kernel<WAVES, UNROLL, GLU, TOut>;
+  // more than 64 KB of dynamic LDS has to be allowed once per kernel (and per process)
+  static const hipError_t allowed =
+      hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
+  if (allowed != hipSuccess) return nhv_fail("few-rows gemm: %s", hipGetErrorString(allowed));
+  const int steps_per_wave = 2 * ((p.pass_steps + 2 * WAVES - 1) / (2 * WAVES));
+  hipLaunchKernelGGL(kernel, dim3(p.grid), dim3(64 * WAVES), p.lds, s, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias,
+                     (TOut*)y, M, N, K, (N + 15) / 16, p.npasses, p.pass_steps, steps_per_wave, p.tiles_per_block);
+  return 0;
+}
+
 struct Plan {
   int nt, waves, unroll;
 };
@@ -454,6 +600,20 @@ int nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* 
   NHV_RESIDENT_CASE(8, 2, false, true)
   NHV_RESIDENT_CASE(8, 8, false, true)
 #undef NHV_RESIDENT_CASE
+  if (rp.waves == 0) {
+    // two pieces of x were faster than the kernel below in all cases but one tie (gate_up at 16 rows of 5,120
+    // columns: 97 against 112 us for 17,408 outputs), three and more pieces slower in most
+    const PassesPlan pp = passes_plan(glu, M, N, K);
+#define NHV_PASSES_CASE(WV_, UN_, GLU_)                                                                  \
+  if (pp.npasses == 2 && pp.waves == WV_ && pp.unroll == UN_ && glu == GLU_)                             \
+    return out_dtype == NHV_BF16 ? launch_passes<WV_, UN_, GLU_, bf16_t>(pp, s, x, w, bias, y, M, N, K)  \
+                                 : launch_passes<WV_, UN_, GLU_, float>(pp, s, x, w, bias, y, M, N, K);
+    NHV_PASSES_CASE(8, 2, true)
+    NHV_PASSES_CASE(4, 8, true)
+    NHV_PASSES_CASE(16, 2, false)
+    NHV_PASSES_CASE(8, 8, false)
+#undef NHV_PASSES_CASE
+  }
   const Plan p = plan(glu, M, N, K);
 #define NHV_FEWROWS_CASE(NT_, WV_, UN_, GLU_)                                              \
   if (p.nt == NT_ && p.waves == WV_ && p.unroll == UN_ && glu == GLU_) {                   \

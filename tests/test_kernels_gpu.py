@@ -140,6 +140,8 @@ def test_skinny_linear_bfloat16(ops, M, N, K):
     (16, 16, 8), (3, 17, 25608),
     # x too large for LDS at once, up to 256 tiles: it comes in pieces
     (16, 4000, 12296), (7, 272, 12288), (11, 4096, 25600),
+    # x too large for LDS at once and more than 256 tiles: two pieces, every tile walked over twice
+    (16, 7168, 5120), (10, 5136, 8200), (5, 4112, 17408),
 ])
 def test_few_rows_linear_bfloat16_in_all_its_variants(ops, M, N, K):
     x = rnd(M, K, dtype=torch.bfloat16, seed=34)
@@ -153,7 +155,7 @@ def test_few_rows_linear_bfloat16_in_all_its_variants(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 112, 80), (5, 1001, 96), (16, 12288, 4096), (17, 160, 96), (64, 300, 1024),
-                                   (4, 17408, 136), (16, 25600, 72), (13, 25000, 264)])
+                                   (4, 17408, 136), (16, 25600, 72), (13, 25000, 264), (16, 9000, 5120), (15, 520, 5384)])
 def test_gated_linear(ops, M, I, K):
     """silu(x Wg^T) * (x Wu^T): the fused kernel for few rows, the two-kernel way for many; float32 as well."""
     for dtype in DTYPES:
