@@ -236,11 +236,15 @@ constexpr int MLPR = MQ <= 4 ? 4 : MQ <= 8 ? 8 : MQ <= 16 ? 16 : MQ <= 32 ? 32 :
 constexpr int MROWS = 64 / MLPR;                            // splits worked on side by side
 constexpr int MPIECES = (MQ + MLPR - 1) / MLPR;             // pieces per lane (more than 1 for heads above 256)
 
-__global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                          bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                                          int window, int split_len, int n_splits, int Hq) {
+// W: waves per (token, head); with many splits and few tokens (one request, 30,000 keys: 235 splits) a single
+// wave's chain of loads is what the merge takes; four waves take every fourth pair of splits and add up through LDS.
+template <int W>
+__global__ __launch_bounds__(64 * W) void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                              bf16_t* __restrict__ out, const int* __restrict__ positions,
+                                                              int window, int split_len, int n_splits, int Hq) {
+  __shared__ float4 sum_s[W > 1 ? W - 1 : 1][MPIECES][64];
   const int item = blockIdx.x;               // t * Hq + h
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int t = item / Hq;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
@@ -259,7 +263,7 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
 #pragma unroll
   for (int i = 0; i < MPIECES; ++i) acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 4
-  for (int s = s0 + sub; s <= s1; s += MROWS) {
+  for (int s = s0 + wave * MROWS + sub; s <= s1; s += MROWS * W) {
     const float wgt = exp2f(ml[s * 2] - m);
 #pragma unroll
     for (int i = 0; i < MPIECES; ++i) {
@@ -277,6 +281,21 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
       acc[i].x += __shfl_xor(acc[i].x, off, 64); acc[i].y += __shfl_xor(acc[i].y, off, 64);
       acc[i].z += __shfl_xor(acc[i].z, off, 64); acc[i].w += __shfl_xor(acc[i].w, off, 64);
     }
+  }
+  if (W > 1) {                               // the other waves' sums, added in the order of the waves
+    if (wave > 0) {
+#pragma unroll
+      for (int i = 0; i < MPIECES; ++i) sum_s[wave - 1][i][lane] = acc[i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int wv = 0; wv < W - 1; ++wv)
+#pragma unroll
+      for (int i = 0; i < MPIECES; ++i) {
+        const float4 v = sum_s[wv][i][lane];
+        acc[i].x += v.x; acc[i].y += v.y; acc[i].z += v.z; acc[i].w += v.w;
+      }
   }
   if (sub == 0) {
 #pragma unroll
@@ -316,8 +335,14 @@ extern "C" int nhv_decode_attention_bf16(const void* q, const void* k_cache, con
                      (const int*)positions, (const int*)block_tables, max_blocks, Hq, Hkv, page_size, page_shift,
                      scale * 1.4426950408889634f, window, split_len, n_splits);
   NHV_LAUNCH_CHECK("decode_attention");
-  hipLaunchKernelGGL(merge_splits_kernel, dim3((unsigned)((size_t)T * Hq)), dim3(64), 0, s, (const float*)part_o,
-                     (const float*)part_ml, (bf16_t*)out, (const int*)positions, window, split_len, n_splits, Hq);
+  // (what decides is the number of splits the launch is made for: inside a graph that is the bound's, but few
+  // tokens with a bound of many splits are the case where the four waves pay, and otherwise they cost nothing much)
+  if (n_splits > 32 && (size_t)T * Hq <= 1024)
+    hipLaunchKernelGGL(merge_splits_kernel<4>, dim3((unsigned)((size_t)T * Hq)), dim3(256), 0, s, (const float*)part_o,
+                       (const float*)part_ml, (bf16_t*)out, (const int*)positions, window, split_len, n_splits, Hq);
+  else
+    hipLaunchKernelGGL(merge_splits_kernel<1>, dim3((unsigned)((size_t)T * Hq)), dim3(64), 0, s, (const float*)part_o,
+                       (const float*)part_ml, (bf16_t*)out, (const int*)positions, window, split_len, n_splits, Hq);
   NHV_LAUNCH_CHECK("merge_splits");
   return 0;
 }

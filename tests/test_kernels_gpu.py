@@ -326,6 +326,18 @@ def test_decode_attention_bfloat16(ops, Hq, Hkv, D, page, window):
     torch.testing.assert_close(one.float(), out[9:10].float(), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(8, 2, 128, 256, None), (6, 1, 48, 16, None), (4, 4, 64, 64, 3000)])
+def test_decode_attention_of_few_tokens_over_many_splits(ops, Hq, Hkv, D, page, window):
+    """One or two requests of thousands of keys: more than 32 splits of 64 keys, which four waves merge."""
+    for lens in ([5000], [4097, 2100]):
+        q_lens = [1] * len(lens)
+        scale = D ** -0.5
+        q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=27, scale=1.5)
+        out = ops.paged_attention(q, kc, vc, batch, bt, scale, window)
+        ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, window)
+        torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("Hq,Hkv,D,page,window", [
     (4, 1, 128, 256, None), (8, 2, 64, 16, None), (6, 1, 32, 8, 100), (3, 3, 48, 5, None), (16, 1, 16, 64, None),
     (5, 1, 256, 32, None), (32, 8, 128, 64, 700),
