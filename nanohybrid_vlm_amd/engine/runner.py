@@ -443,8 +443,13 @@ class ModelRunner:
             eager = self.model.logits(self.model.forward(ctx)).clone()
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                logits = self.model.logits(self.model.forward(ctx))
+            try:
+                with torch.cuda.graph(graph):
+                    logits = self.model.logits(self.model.forward(ctx))
+            except RuntimeError as err:                       # something in the step cannot be recorded
+                print(f"[nanohybrid_vlm_amd] no graph for {bucket} requests ({str(err).splitlines()[0][:200]}); "
+                      "steps of this size run eagerly", file=sys.stderr, flush=True)
+                return {"graph": None, "index": index, "logits": eager, "ctx": ctx, "planned": planned}
             if with_library:
                 for _ in range(3):
                     logits.fill_(float("nan"))
