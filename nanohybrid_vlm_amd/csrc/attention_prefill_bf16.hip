@@ -184,8 +184,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     return BT_IN_LDS ? slot_of((const int*)bt_s, key, page_size, page_shift) : slot_of(bt_g, key, page_size, page_shift);
   };
 
-  // memory -> LDS without registers: wave w's load number i brings pieces (4 i + w) * 64 + lane of the tile
+  // memory -> LDS without registers: wave w's load number i brings pieces (4 i + w) * 64 + lane of the tile.
+  // With pages that are a power of two and hold whole tiles, a tile inside the block's key range lies in one page
+  // at a place that is the same for the whole block: one look-up and scalar arithmetic, and each thread adds
+  // offsets that it worked out once. Other tiles (the range's ends, other page sizes) look every key up.
+  const bool whole_tiles = page_shift >= 0 && page_size >= BN;
+  int k_off[LOADS], v_off[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int u = (i * 4 + wave) * 64 + lane;
+    const int kl = u / CH, piece = u % CH;
+    k_off[i] = (kl * Hkv + kvh) * D + (piece ^ (kl & KSWZ)) * 8;
+    v_off[i] = (kl * Hkv + kvh) * D + (piece ^ ((kl & VSWZ) << 1)) * 8;
+  }
   auto issue = [&](int kb, bf16_t* k_s, bf16_t* v_s) {
+    if (whole_tiles && kb >= key_lo && kb + BN - 1 <= key_hi) {
+      const int page = __builtin_amdgcn_readfirstlane(BT_IN_LDS ? bt_s[kb >> page_shift] : bt_g[kb >> page_shift]);
+      const size_t tile_off = (((size_t)page << page_shift) + (kb & (page_size - 1))) * Hkv * D;
+      const bf16_t* k_tile = k_cache + tile_off;
+      const bf16_t* v_tile = v_cache + tile_off;
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i)
+        if (PIECES % 256 == 0 || (i * 4 + wave) * 64 + lane < PIECES) {
+          __builtin_amdgcn_global_load_lds((global_ptr)(k_tile + k_off[i]), (lds_ptr)(k_s + (i * 4 + wave) * 512), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((global_ptr)(v_tile + v_off[i]), (lds_ptr)(v_s + (i * 4 + wave) * 512), 16, 0, 0);
+        }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int u = (i * 4 + wave) * 64 + lane;
