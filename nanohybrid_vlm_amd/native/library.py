@@ -55,14 +55,14 @@ def _sources(names: list[str]) -> list[str]:
     return [os.path.join(CSRC, n) for n in names]
 
 
-def _digest(sources: list[str], defines: list[str]) -> str:
+def _digest(sources: list[str], defines: list[str], link: list[str] | None = None) -> str:
     h = hashlib.sha256()
     for path in sorted(sources) + sorted(
             os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")):
         h.update(os.path.basename(path).encode())
         with open(path, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(HIPCC_FLAGS + defines).encode())
+    h.update(" ".join(HIPCC_FLAGS + defines + list(link or [])).encode())
     return h.hexdigest()[:16]
 
 
@@ -93,11 +93,14 @@ def _compile_one(src: str, obj: str, defines: list[str]) -> None:
     _say(f"compiled {os.path.basename(src)} {' '.join(defines)} in {time.time() - t0:.1f} s")
 
 
-def build_library(stem: str, source_names: list[str], defines: list[str] | None = None, force: bool = False) -> str:
-    """Compile ``source_names`` into ``lib<stem>_<hash>.so`` and return its path."""
+def build_library(stem: str, source_names: list[str], defines: list[str] | None = None, force: bool = False,
+                  link: list[str] | None = None) -> str:
+    """Compile ``source_names`` into ``lib<stem>_<hash>.so`` and return its path. ``link``: further arguments of the
+    link step (libraries the sources call)."""
     defines = list(defines or [])
+    link = list(link or [])
     sources = _sources(source_names)
-    file_name = f"lib{stem}_{_digest(sources, defines)}.so"
+    file_name = f"lib{stem}_{_digest(sources, defines, link)}.so"
     if not force:
         for path in _candidates(file_name):
             if os.path.isfile(path):
@@ -111,7 +114,7 @@ def build_library(stem: str, source_names: list[str], defines: list[str] | None 
         with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
             list(pool.map(lambda so: _compile_one(so[0], so[1], defines), zip(sources, objs)))
         tmp_target = os.path.join(work, file_name)
-        cmd = [_hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc", *objs, "-o", tmp_target]
+        cmd = [_hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc", *objs, *link, "-o", tmp_target]
         proc = subprocess.run(cmd, capture_output=True, text=True)
         if proc.returncode != 0:
             raise NativeBuildError(f"linking {file_name} failed:\n{proc.stderr[-4000:]}")
@@ -132,11 +135,12 @@ def build_library(stem: str, source_names: list[str], defines: list[str] | None 
 _loaded: dict[str, ctypes.CDLL] = {}
 
 
-def load_library(stem: str, source_names: list[str], defines: list[str] | None = None) -> ctypes.CDLL:
+def load_library(stem: str, source_names: list[str], defines: list[str] | None = None,
+                 link: list[str] | None = None) -> ctypes.CDLL:
     key = stem + "|" + " ".join(defines or [])
     lib = _loaded.get(key)
     if lib is None:
-        path = build_library(stem, source_names, defines)
+        path = build_library(stem, source_names, defines, link=link)
         lib = ctypes.CDLL(path)
         _loaded[key] = lib
     return lib

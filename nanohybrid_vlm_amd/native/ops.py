@@ -20,10 +20,13 @@ from . import library
 
 CORE_SOURCES = ["error.hip", "elementwise.hip", "gemm_generic.hip", "gemm_skinny_bf16.hip", "gemm_fewrows_bf16.hip", "attention_generic.hip",
                 "sampling.hip"]
+BLAS_SOURCES = ["error.hip", "gemm_library.hip"]                                                   # the vendor's matrix library, algorithm by number
+BLAS_LINK = ["-lhipblaslt"]
 ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip", "attention_prefill_bf16.hip"]      # compiled once per head size
 ATTENTION_HEAD_DIMS_BUILT_AHEAD = [16, 32, 48, 64, 80, 96, 112, 128, 256]
 
 F32, BF16 = 0, 1
+OWN = -1      # a measured choice for a matrix product: the own kernel (0, 1, ...: that algorithm of the library's list)
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -93,10 +96,13 @@ class NativeBackend:
 
     name = "hip"
     device_type = "cuda"
-    few_rows = 16                 # up to this many rows the own matrix kernels are the faster ones
+    few_rows = 16                 # up to this many rows the own matrix kernels are the rule
+    library_rows = 64             # up to this many rows the way a product is done may be chosen by measurement (see _choose)
+    library_algorithms = 48       # so many of the library's algorithms are asked for and tried
+    library_workspace = 32 << 20  # bytes of scratch memory the library's algorithms may use
     own_kernels_only = False      # True: no library call (matrix products of up to 64 rows take the own kernels)
     planned_context = 0           # > 0 while a HIP graph is recorded: the lengths to plan for (the batch's own are bounds)
-    measure_linears = False       # True: a few-rows product of a shape not seen before is timed both ways (see linear)
+    measure_linears = False       # True: a product of few rows and a shape not seen before is timed in every way there is (see _choose)
 
     def __init__(self):
         if not torch.cuda.is_available():
@@ -104,7 +110,10 @@ class NativeBackend:
         self.lib = library.load_library("nhv_core", CORE_SOURCES)
         self.lib.nhv_last_error.restype = ctypes.c_char_p
         self._attention_libs: dict[int, ctypes.CDLL] = {}
-        self.library_is_faster: dict[tuple, bool] = {}     # (M, N, K, gated) of few-rows products -> measured
+        self.chosen: dict[tuple, int] = {}                  # (M, N, K, float result, gated) of a product -> OWN or a library algorithm, measured
+        self._blas = None
+        self._plans: dict[tuple, tuple[int, int]] = {}
+        self._workspace = None
         self._sweep = None                                  # scratch memory whose writing empties the caches before a measurement
 
     def _call(self, fn_name: str, *args, lib=None) -> None:
@@ -187,66 +196,120 @@ class NativeBackend:
                    block_tables.shape[1], T, Hq, Hkv, page_size, ctypes.c_float(scale), window, split_len, n_splits,
                    _stream(), lib=self.attention_lib(D))
 
-    def _faster(self, first, second, what: str) -> bool:
-        """Whether ``second()`` takes less than 0.95 of the time of ``first()`` on the GPU. Each is timed five times,
-        alone and after a write of 512 MB has swept the caches (the memory-side one holds 256 MB): in a decoding
-        step a weight comes from memory, and a weight left in a cache by the run before would be measured 15 to
-        20 % too fast, by an amount that differs between the two."""
-        if self._sweep is None:
-            try:
-                self._sweep = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
-            except torch.OutOfMemoryError:
-                return False                                 # no room to measure: the own kernel, as the rule says
-        best = []
-        for run in (first, second):
-            run()                                            # loads what the call needs
-            times = []
-            for _ in range(5):
-                self._sweep.zero_()
-                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                start.record()
-                run()
-                end.record()
-                end.synchronize()
-                times.append(start.elapsed_time(end))
-            best.append(min(times))
-        if os.environ.get("NHV_SHOW_MEASUREMENTS"):
-            print(f"[nanohybrid_vlm_amd] {what}: own {1e3 * best[0]:.1f} us, library {1e3 * best[1]:.1f} us",
-                  file=sys.stderr, flush=True)
-        return best[1] < 0.95 * best[0]
+    # -- matrix products of few rows: own kernel or one of the library's algorithms, by measurement --
+    def blas_lib(self) -> ctypes.CDLL:
+        """The wrapper of the vendor's matrix library, loaded when a product is first given to it."""
+        if self._blas is None:
+            self._blas = library.load_library("nhv_blas", BLAS_SOURCES, link=BLAS_LINK)
+            self._blas.nhv_last_error.restype = ctypes.c_char_p
+        return self._blas
 
-    def _few_rows_by_library(self, x, w, out, gated: bool = False) -> bool:
-        """Whether this product of up to ``few_rows`` rows goes to the library (``gated``: followed by the
-        SiLU-and-multiply kernel, instead of the own kernel that does both). The own kernel is the rule; which
-        of the two is faster depends on the shape in ways no rule here captures (at 8 rows the library takes 21
-        against 25 us for a 4096 x 12288 matrix and 112 against 50 us for a 5120 x 17408 one), so while
-        ``measure_linears`` is set (the run before a graph is recorded) a shape not seen before is timed both
-        ways, and the answer is kept for the life of the process."""
+    def _library_plan(self, M: int, N: int, K: int, float_result: bool) -> tuple[int, int]:
+        """(plan, number of algorithms) of the library for this shape."""
+        key = (M, N, K, float_result)
+        got = self._plans.get(key)
+        if got is None:
+            plan, count = ctypes.c_int(), ctypes.c_int()
+            self._call("nhv_library_gemm_plan", M, N, K, F32 if float_result else BF16, self.library_algorithms,
+                       ctypes.c_size_t(self.library_workspace), ctypes.byref(plan), ctypes.byref(count), lib=self.blas_lib())
+            got = self._plans[key] = (plan.value, count.value)
+        return got
+
+    def _library_product(self, x, w, out, algorithm: int) -> None:
+        plan, _ = self._library_plan(x.shape[0], w.shape[0], x.shape[1], out.dtype == torch.float32)
+        if self._workspace is None:
+            self._workspace = torch.empty(self.library_workspace, dtype=torch.uint8, device=x.device)
+        self._call("nhv_library_gemm", plan, algorithm, _ptr(x), _ptr(w), _ptr(out), _ptr(self._workspace),
+                   ctypes.c_size_t(self.library_workspace), _stream(), lib=self.blas_lib())
+
+    def _time_cold(self, run, repeats: int) -> float:
+        """The shortest of ``repeats`` runs in milliseconds, each alone and after a read of 512 MB has swept the
+        caches (the memory-side one holds 256 MB): in a decoding step a weight comes from memory, and a weight
+        left in a cache by the run before would be measured 15 to 20 % too fast, by an amount that differs from
+        kernel to kernel. The sweep reads, as the step before a product does: after a sweep that writes, the
+        caches are full of lines that have to go back to memory while the product runs, which adds 10 to 35 us."""
+        times = []
+        for _ in range(repeats):
+            self._sweep.sum()
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            run()
+            end.record()
+            end.synchronize()
+            times.append(start.elapsed_time(end))
+        return min(times)
+
+    def _choose(self, x, w, out, gated: bool = False) -> int | None:
+        """How this product of up to ``library_rows`` rows is done: ``OWN`` (the own kernel; with ``gated`` the one
+        that also does the SiLU-and-multiply), the number of one of the library's algorithms (``gated``: followed by
+        the SiLU-and-multiply kernel), or ``None`` if the shape was never measured (then the rule holds: own kernel up
+        to ``few_rows`` rows, the library's first guess above). Which is fastest depends on the shape in ways no rule
+        here captures, and the library's own first guess is often far from its best (a 5120 x 17408 weight against 8
+        rows: 112 us by its first guess, 37 us by another of its algorithms, 50 us by the own kernel; a 4096 x 12288
+        weight: 22, 22 and 25 us). So while ``measure_linears`` is set (the run before a graph is recorded) a shape
+        not seen before is timed in every way there is, and the answer is kept for the life of the process. An
+        algorithm whose result differs from the own kernel's by more than rounding, or from its own on a second
+        run, is left out. The own kernel stays unless a library algorithm takes less than 0.95 of its time."""
         M, K = x.shape
         N = w.shape[0]
-        key = (M, N, K, gated)
-        known = self.library_is_faster.get(key)
+        float_result = out.dtype == torch.float32
+        key = (M, N, K, float_result, gated)
+        known = self.chosen.get(key)
         if known is not None or not self.measure_linears or torch.cuda.is_current_stream_capturing():
-            return bool(known)
-        if gated:
-            packed = torch.empty((M, N), dtype=x.dtype, device=x.device)
+            return known
+        if self._sweep is None:
+            try:
+                self._sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
+            except torch.OutOfMemoryError:
+                return None                                  # no room to measure: the rule
+        packed = torch.empty((M, N), dtype=x.dtype, device=x.device) if gated else out
 
-            def own():
+        def own():
+            if gated:
                 self._call("nhv_gemm_skinny_glu_bf16", _ptr(x), _ptr(w), _ptr(out), M, N // 2, K, dtype_code(out), _stream())
-
-            def library():
-                torch.mm(x, w.t(), out=packed)
-                self.silu_mul(packed, out)
-        else:
-            def own():
+            else:
                 self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), None, _ptr(out), M, N, K, dtype_code(out), _stream())
 
-            def library():
-                torch.mm(x, w.t(), out=out)
-        self.library_is_faster[key] = self._faster(own, library, f"{'gated ' if gated else ''}product {M} x {K} . {N} x {K}")
-        if gated and self.library_is_faster[key]:
-            self.library_is_faster[(M, N, K, False)] = True  # the packed product that follows a refusal of gated_linear
-        return self.library_is_faster[key]
+        def by_library(algorithm):
+            def run():
+                self._library_product(x, w, packed, algorithm)
+                if gated:
+                    self.silu_mul(packed, out)
+            return run
+
+        own()
+        reference = out.float()
+        bound = (1e-3 if float_result else 2e-2) * max(float(reference.abs().max()), 1e-30)
+        runs = {OWN: own} if M <= self.few_rows else {}
+        _, count = self._library_plan(M, N, K, float_result and not gated)
+        for algorithm in range(count):
+            run = by_library(algorithm)
+            try:
+                out.zero_()
+                run()
+                first = out.clone()
+                out.zero_()
+                run()
+            except KernelError:
+                continue
+            if torch.equal(first, out) and float((out.float() - reference).abs().max()) <= bound:
+                runs[algorithm] = run
+        once = sorted((self._time_cold(run, 1), how) for how, run in runs.items())
+        best = sorted((min(t, self._time_cold(runs[how], 4)), how) for t, how in once[:4])
+        how = best[0][1]
+        own_time = next((t for t, h in best if h == OWN), None) or next((t for t, h in once if h == OWN), None)
+        if own_time is not None and how != OWN and best[0][0] >= 0.95 * own_time:
+            how = OWN
+        if os.environ.get("NHV_SHOW_MEASUREMENTS"):
+            first_guess = next((t for t, h in once if h == 0), float("nan"))
+            print(f"[nanohybrid_vlm_amd] {'gated ' if gated else ''}product {M} x {K} . {N} x {K}: own "
+                  f"{'-' if own_time is None else format(1e3 * own_time, '.1f')} us, library's first guess "
+                  f"{1e3 * first_guess:.1f} us, fastest {1e3 * best[0][0]:.1f} us ({'own' if best[0][1] == OWN else best[0][1]} "
+                  f"of {len(runs)} ways); taken: {'own' if how == OWN else how}", file=sys.stderr, flush=True)
+        self.chosen[key] = how
+        if gated and how != OWN:
+            self.chosen[(M, N, K, False, False)] = how       # the packed product that follows a refusal of gated_linear
+        return how
 
     def end_measurements(self) -> None:
         """Gives the scratch memory of the measurements back (what was measured stays known)."""
@@ -256,10 +319,10 @@ class NativeBackend:
         M, K = x.shape
         N = w.shape[0]
         if x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
-            if M <= self.few_rows and out.dtype == torch.bfloat16 and bias is None and not self.own_kernels_only \
-                    and self._few_rows_by_library(x, w, out):
-                torch.mm(x, w.t(), out=out)
-                return None
+            if M <= self.library_rows and bias is None and not self.own_kernels_only:
+                how = self._choose(x, w, out)
+                if how is not None and how != OWN:
+                    return self._library_product(x, w, out, how)
             if M <= self.few_rows or (M <= 64 and self.own_kernels_only):
                 return self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
                                   dtype_code(out), _stream())
@@ -287,7 +350,7 @@ class NativeBackend:
         M, K = x.shape
         if (x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
                 and (M <= self.few_rows or (M <= 64 and self.own_kernels_only))):
-            if M <= self.few_rows and not self.own_kernels_only and self._few_rows_by_library(x, w, out, gated=True):
+            if M <= self.few_rows and not self.own_kernels_only and self._choose(x, w, out, gated=True) not in (None, OWN):
                 return False                                 # the library's product, then silu_mul
             self._call("nhv_gemm_skinny_glu_bf16", _ptr(x), _ptr(w), _ptr(out), M, out.shape[1], K, dtype_code(out),
                        _stream())

@@ -458,34 +458,43 @@ def test_refusals(ops):
         ops.rmsnorm(torch.zeros(2, 8), torch.ones(8), 1e-6)
 
 
-def test_few_rows_products_are_given_to_the_faster_of_own_kernel_and_library(ops):
-    """While ``measure_linears`` is set a shape not seen before is timed both ways and the answer kept; whichever
-    way a product goes, it is the same product."""
+def test_products_of_few_rows_are_done_the_fastest_way_measured(ops):
+    """While ``measure_linears`` is set a shape not seen before is timed by the own kernel and by every algorithm
+    of the library, and the answer kept; whichever way a product goes, it is the same product."""
+    from nanohybrid_vlm_amd.native.ops import OWN
     backend = ops.backend()
-    M, N, K = 8, 512, 1024
-    x = rnd(M, K, dtype=torch.bfloat16, seed=51)
-    w = rnd(N, K, dtype=torch.bfloat16, seed=52, scale=K ** -0.5)
-    w2 = rnd(2 * N, K, dtype=torch.bfloat16, seed=53, scale=K ** -0.5)
-    ref = x.double() @ w.double().T
-    g, u = x.double() @ w2[:N].double().T, x.double() @ w2[N:].double().T
-    keys = [(M, N, K, False), (M, 2 * N, K, True)]
-    saved = {k: backend.library_is_faster.pop(k, None) for k in keys + [(M, 2 * N, K, False)]}
-    try:
-        assert ops.linear(x, w) is not None and keys[0] not in backend.library_is_faster      # not measured unasked
-        backend.measure_linears = True
+    N, K = 512, 1024
+    for M in (8, 40):                                       # the own kernel is among the ways / the library's ways only
+        x = rnd(M, K, dtype=torch.bfloat16, seed=51)
+        w = rnd(N, K, dtype=torch.bfloat16, seed=52, scale=K ** -0.5)
+        w2 = rnd(2 * N, K, dtype=torch.bfloat16, seed=53, scale=K ** -0.5)
+        ref = x.double() @ w.double().T
+        g, u = x.double() @ w2[:N].double().T, x.double() @ w2[N:].double().T
+        keys = [(M, N, K, False, False), (M, N, K, True, False)] + ([(M, 2 * N, K, False, True)] if M <= 16 else [])
+        every = keys + [(M, 2 * N, K, False, False)]
+        saved = {k: backend.chosen.pop(k, None) for k in every}
         try:
-            ops.linear(x, w)
-            ops.gated_linear(x, w2)
+            assert ops.linear(x, w) is not None and keys[0] not in backend.chosen      # not measured unasked
+            backend.measure_linears = True
+            try:
+                ops.linear(x, w)
+                ops.linear(x, w, out_dtype=torch.float32)
+                ops.gated_linear(x, w2)
+            finally:
+                backend.measure_linears = False
+                backend.end_measurements()
+            assert all(isinstance(backend.chosen[k], int) for k in keys)
+            assert M <= 16 or all(backend.chosen[k] != OWN for k in keys)
+            _, count = backend._library_plan(M, N, K, False)
+            assert count > 0
+            for how in [OWN] + list(range(min(count, 3))):
+                for k in every:
+                    backend.chosen[k] = how
+                torch.testing.assert_close(ops.linear(x, w).double(), ref, **tol(torch.bfloat16))
+                torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32).double(), ref, rtol=1e-4, atol=1e-4)
+                torch.testing.assert_close(ops.gated_linear(x, w2).double(), g * torch.sigmoid(g) * u, **tol(torch.bfloat16))
         finally:
-            backend.measure_linears = False
-        assert all(isinstance(backend.library_is_faster[k], bool) for k in keys)
-        for by_library in (False, True):
-            for k in keys + [(M, 2 * N, K, False)]:
-                backend.library_is_faster[k] = by_library
-            torch.testing.assert_close(ops.linear(x, w).double(), ref, **tol(torch.bfloat16))
-            torch.testing.assert_close(ops.gated_linear(x, w2).double(), g * torch.sigmoid(g) * u, **tol(torch.bfloat16))
-    finally:
-        for k, v in saved.items():
-            backend.library_is_faster.pop(k, None)
-            if v is not None:
-                backend.library_is_faster[k] = v
+            for k, v in saved.items():
+                backend.chosen.pop(k, None)
+                if v is not None:
+                    backend.chosen[k] = v
