@@ -368,6 +368,10 @@ class ModelRunner:
             if self._graphs.get(bucket, ...) is not None:
                 return self._graph_step(entries, bucket)
         ctx, new_lens = self.build_context(entries)
+        if self.device.type == "cuda":
+            from ..native import ops
+            backend = ops.backend()
+            backend.step_number = getattr(backend, "step_number", 0) + 1      # (shapes that come again, step after step, are measured)
         hidden = self.model.forward(ctx)
         logits = self.model.logits(hidden) if hidden is not None else None
         for e, n in zip(entries, new_lens):

@@ -26,7 +26,8 @@ ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip", "attention_prefil
 ATTENTION_HEAD_DIMS_BUILT_AHEAD = [16, 32, 48, 64, 80, 96, 112, 128, 256]
 
 F32, BF16 = 0, 1
-OWN = -1      # a measured choice for a matrix product: the own kernel (0, 1, ...: that algorithm of the library's list)
+# a measured choice for a matrix product: the own kernel, or what the rule gives (0, 1, ...: that algorithm of the library's list)
+OWN, RULE = -1, -2
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -103,6 +104,8 @@ class NativeBackend:
     own_kernels_only = False      # True: no library call (matrix products of up to 64 rows take the own kernels)
     planned_context = 0           # > 0 while a HIP graph is recorded: the lengths to plan for (the batch's own are bounds)
     measure_linears = False       # True: a product of few rows and a shape not seen before is timed in every way there is (see _choose)
+    measure_many_rows = True      # a product of more than library_rows rows is timed in the third step that meets its shape
+    step_number = 0               # counted by the engine, one per eager step
 
     def __init__(self):
         if not torch.cuda.is_available():
@@ -113,6 +116,7 @@ class NativeBackend:
         self.chosen: dict[tuple, int] = {}                  # (M, N, K, float result, gated) of a product -> OWN or a library algorithm, measured
         self._blas = None
         self._plans: dict[tuple, tuple[int, int]] = {}
+        self._met: dict[tuple, tuple[int, int]] = {}        # shape of many rows -> (steps that met it, the last of them)
         self._workspace = None
         self._sweep = None                                  # scratch memory whose writing empties the caches before a measurement
 
@@ -240,32 +244,59 @@ class NativeBackend:
         return min(times)
 
     def _choose(self, x, w, out, gated: bool = False) -> int | None:
-        """How this product of up to ``library_rows`` rows is done: ``OWN`` (the own kernel; with ``gated`` the one
-        that also does the SiLU-and-multiply), the number of one of the library's algorithms (``gated``: followed by
-        the SiLU-and-multiply kernel), or ``None`` if the shape was never measured (then the rule holds: own kernel up
-        to ``few_rows`` rows, the library's first guess above). Which is fastest depends on the shape in ways no rule
-        here captures, and the library's own first guess is often far from its best (a 5120 x 17408 weight against 8
-        rows: 112 us by its first guess, 37 us by another of its algorithms, 50 us by the own kernel; a 4096 x 12288
-        weight: 22, 22 and 25 us). So while ``measure_linears`` is set (the run before a graph is recorded) a shape
-        not seen before is timed in every way there is, and the answer is kept for the life of the process. An
-        algorithm whose result differs from the own kernel's by more than rounding, or from its own on a second
-        run, is left out. The own kernel stays unless a library algorithm takes less than 0.95 of its time."""
+        """How this product is done: ``OWN`` (the own kernel; with ``gated`` the one that also does the
+        SiLU-and-multiply), the number of one of the library's algorithms (``gated``: followed by the
+        SiLU-and-multiply kernel), ``RULE`` (measured, and nothing beat what the rule gives), or ``None`` if the
+        shape was never measured (then the rule holds too: own kernel up to ``few_rows`` rows, ``torch.mm`` above).
+        Which is fastest depends on the shape in ways no rule here captures, and the library's own first guess is
+        often far from its best (a 5120 x 17408 weight against 8 rows: 112 us by its first guess, 37 us by another
+        of its algorithms, 50 us by the own kernel; a 4096 x 12288 weight: 22, 22 and 25 us; the same weight
+        against 2,048 rows: 197 us by ``torch.mm``, 173 us by the library's second guess). So a shape is timed in
+        every way there is, once, and the answer is kept for the life of the process: a shape of up to
+        ``library_rows`` rows while ``measure_linears`` is set (the run before a graph is recorded), a shape of
+        more rows (a portion of a prompt) in the third step that meets it, since only the sizes that come again
+        and again (portions that fill the token budget) are worth the 50 ms. An algorithm whose result differs
+        from the trusted way's (own kernel, ``torch.mm``) by more than rounding, or from its own on a second run,
+        is left out. The trusted way stays unless a library algorithm takes less than 0.95 of its time."""
         M, K = x.shape
         N = w.shape[0]
         float_result = out.dtype == torch.float32
         key = (M, N, K, float_result, gated)
         known = self.chosen.get(key)
-        if known is not None or not self.measure_linears or torch.cuda.is_current_stream_capturing():
+        if known is not None or torch.cuda.is_current_stream_capturing():
             return known
+        many = M > self.library_rows
+        if many:
+            met, step = self._met.get(key, (0, -1))
+            if step != self.step_number:                     # (a model's layers meet the same shape in one step)
+                met += 1
+                self._met[key] = (met, self.step_number)
+            if not self.measure_many_rows or met < 3:
+                return None
+        elif not self.measure_linears:
+            return None
+        try:
+            how = self._measure(x, w, out, gated, many)
+        except torch.OutOfMemoryError:
+            how = RULE if many else None                     # no room to measure: the rule
+        if how is not None:
+            self.chosen[key] = how
+            if gated and how >= 0:
+                self.chosen[(M, N, K, False, False)] = how   # the packed product that follows a refusal of gated_linear
+        return how
+
+    def _measure(self, x, w, out, gated: bool, many: bool) -> int:
+        M, K = x.shape
+        N = w.shape[0]
+        float_result = out.dtype == torch.float32
         if self._sweep is None:
-            try:
-                self._sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
-            except torch.OutOfMemoryError:
-                return None                                  # no room to measure: the rule
+            self._sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
         packed = torch.empty((M, N), dtype=x.dtype, device=x.device) if gated else out
 
-        def own():
-            if gated:
+        def trusted():
+            if many:
+                torch.mm(x, w.t(), out=out)
+            elif gated:
                 self._call("nhv_gemm_skinny_glu_bf16", _ptr(x), _ptr(w), _ptr(out), M, N // 2, K, dtype_code(out), _stream())
             else:
                 self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), None, _ptr(out), M, N, K, dtype_code(out), _stream())
@@ -277,12 +308,13 @@ class NativeBackend:
                     self.silu_mul(packed, out)
             return run
 
-        own()
-        reference = out.float()
+        trusted()
+        reference = out.clone()
         bound = (1e-3 if float_result else 2e-2) * max(float(reference.abs().max()), 1e-30)
-        runs = {OWN: own} if M <= self.few_rows else {}
+        incumbent = RULE if many else OWN
+        runs = {incumbent: trusted} if many or M <= self.few_rows else {}
         _, count = self._library_plan(M, N, K, float_result and not gated)
-        for algorithm in range(count):
+        for algorithm in range(min(count, 16) if many else count):
             run = by_library(algorithm)
             try:
                 out.zero_()
@@ -292,23 +324,24 @@ class NativeBackend:
                 run()
             except KernelError:
                 continue
-            if torch.equal(first, out) and float((out.float() - reference).abs().max()) <= bound:
+            if torch.equal(first, out) and float((out - reference).abs().max()) <= bound:
                 runs[algorithm] = run
+            del first
         once = sorted((self._time_cold(run, 1), how) for how, run in runs.items())
         best = sorted((min(t, self._time_cold(runs[how], 4)), how) for t, how in once[:4])
         how = best[0][1]
-        own_time = next((t for t, h in best if h == OWN), None) or next((t for t, h in once if h == OWN), None)
-        if own_time is not None and how != OWN and best[0][0] >= 0.95 * own_time:
-            how = OWN
+        incumbent_time = next((t for t, h in best + once if h == incumbent), None)
+        if incumbent_time is not None and how != incumbent and best[0][0] >= 0.95 * incumbent_time:
+            how = incumbent
         if os.environ.get("NHV_SHOW_MEASUREMENTS"):
+            name = {OWN: "own", RULE: "torch.mm"}
             first_guess = next((t for t, h in once if h == 0), float("nan"))
-            print(f"[nanohybrid_vlm_amd] {'gated ' if gated else ''}product {M} x {K} . {N} x {K}: own "
-                  f"{'-' if own_time is None else format(1e3 * own_time, '.1f')} us, library's first guess "
-                  f"{1e3 * first_guess:.1f} us, fastest {1e3 * best[0][0]:.1f} us ({'own' if best[0][1] == OWN else best[0][1]} "
-                  f"of {len(runs)} ways); taken: {'own' if how == OWN else how}", file=sys.stderr, flush=True)
-        self.chosen[key] = how
-        if gated and how != OWN:
-            self.chosen[(M, N, K, False, False)] = how       # the packed product that follows a refusal of gated_linear
+            print(f"[nanohybrid_vlm_amd] {'gated ' if gated else ''}product {M} x {K} . {N} x {K}: {name[incumbent]} "
+                  f"{'-' if incumbent_time is None else format(1e3 * incumbent_time, '.1f')} us, library's first guess "
+                  f"{1e3 * first_guess:.1f} us, fastest {1e3 * best[0][0]:.1f} us ({name.get(best[0][1], best[0][1])} "
+                  f"of {len(runs)} ways); taken: {name.get(how, how)}", file=sys.stderr, flush=True)
+        if many:
+            self._sweep = None                               # (a step of prompt portions is followed by no end_measurements)
         return how
 
     def end_measurements(self) -> None:
@@ -319,9 +352,9 @@ class NativeBackend:
         M, K = x.shape
         N = w.shape[0]
         if x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
-            if M <= self.library_rows and bias is None and not self.own_kernels_only:
+            if bias is None and not self.own_kernels_only and (M <= self.library_rows or out.dtype == torch.bfloat16):
                 how = self._choose(x, w, out)
-                if how is not None and how != OWN:
+                if how is not None and how >= 0:
                     return self._library_product(x, w, out, how)
             if M <= self.few_rows or (M <= 64 and self.own_kernels_only):
                 return self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
@@ -350,8 +383,10 @@ class NativeBackend:
         M, K = x.shape
         if (x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
                 and (M <= self.few_rows or (M <= 64 and self.own_kernels_only))):
-            if M <= self.few_rows and not self.own_kernels_only and self._choose(x, w, out, gated=True) not in (None, OWN):
-                return False                                 # the library's product, then silu_mul
+            if M <= self.few_rows and not self.own_kernels_only:
+                how = self._choose(x, w, out, gated=True)
+                if how is not None and how >= 0:
+                    return False                             # the library's product, then silu_mul
             self._call("nhv_gemm_skinny_glu_bf16", _ptr(x), _ptr(w), _ptr(out), M, out.shape[1], K, dtype_code(out),
                        _stream())
             return True

@@ -498,3 +498,34 @@ def test_products_of_few_rows_are_done_the_fastest_way_measured(ops):
                 backend.chosen.pop(k, None)
                 if v is not None:
                     backend.chosen[k] = v
+
+
+def test_a_shape_of_many_rows_is_measured_in_the_third_step_that_meets_it(ops):
+    """Prompt portions: only a shape that comes step after step is timed (against ``torch.mm``, which stays
+    unless one of the library's algorithms is clearly faster); the product is the same product either way."""
+    from nanohybrid_vlm_amd.native.ops import RULE
+    backend = ops.backend()
+    M, N, K = 200, 384, 512
+    x = rnd(M, K, dtype=torch.bfloat16, seed=61)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=62, scale=K ** -0.5)
+    ref = x.double() @ w.double().T
+    key = (M, N, K, False, False)
+    saved = backend.chosen.pop(key, None), backend._met.pop(key, None)
+    try:
+        for step in range(3):
+            backend.step_number += 1
+            for _ in range(4):                               # layers of one step count once
+                torch.testing.assert_close(ops.linear(x, w).double(), ref, **tol(torch.bfloat16))
+            assert (key in backend.chosen) == (step == 2)
+        assert backend.chosen[key] == RULE or backend.chosen[key] >= 0
+        _, count = backend._library_plan(M, N, K, False)
+        for how in [RULE] + list(range(min(count, 3))):
+            backend.chosen[key] = how
+            torch.testing.assert_close(ops.linear(x, w).double(), ref, **tol(torch.bfloat16))
+    finally:
+        backend.chosen.pop(key, None)
+        backend._met.pop(key, None)
+        if saved[0] is not None:
+            backend.chosen[key] = saved[0]
+        if saved[1] is not None:
+            backend._met[key] = saved[1]
