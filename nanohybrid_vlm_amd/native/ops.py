@@ -118,7 +118,7 @@ class NativeBackend:
         self._plans: dict[tuple, tuple[int, int]] = {}
         self._met: dict[tuple, tuple[int, int]] = {}        # shape of many rows -> (steps that met it, the last of them)
         self._workspace = None
-        self._sweep = None                                  # scratch memory whose writing empties the caches before a measurement
+        self._sweep = None                                  # scratch memory whose reading empties the caches before a measurement
 
     def _call(self, fn_name: str, *args, lib=None) -> None:
         lib = lib or self.lib
@@ -290,7 +290,7 @@ class NativeBackend:
         N = w.shape[0]
         float_result = out.dtype == torch.float32
         if self._sweep is None:
-            self._sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
+            self._sweep = torch.zeros(128 << 20, dtype=torch.float32, device="cuda")      # (a sum of floats is one kernel and no copy)
         packed = torch.empty((M, N), dtype=x.dtype, device=x.device) if gated else out
 
         def trusted():
