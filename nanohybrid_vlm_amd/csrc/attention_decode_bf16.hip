@@ -74,7 +74,11 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
   // blocks go to the eight XCDs in turn by their linear index: with the split as the slowest index every XCD
   // gets the same share of each split (the last splits of a request are short or empty: as the fastest index,
   // four splits a request put all the long ones on half of the chip, 141 us against 108 us at 64 requests)
-  const int kvh = blockIdx.x, t = blockIdx.y, split = blockIdx.z;
+  // and the key/value head turns with the token and the split: a head's keys are 2 D bytes out of every
+  // 2 D Hkv bytes of a page, and an XCD that read one and the same head for every token took 4 to 5 % longer at
+  // 32 and 64 requests (116 against 111 us at 64) than one whose blocks go over all heads
+  const int t = blockIdx.y, split = blockIdx.z;
+  const int kvh = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
   const int G = Hq / Hkv;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
