@@ -168,7 +168,7 @@ class LLM:
             m = self._metrics[seq.seq_id]
             if m.first_scheduled is None:
                 m.first_scheduled = t0
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, keep=False)          # sampled from at once
         tokens_by_id = {}
         if sampled_rows:
             seed = self.config.seed

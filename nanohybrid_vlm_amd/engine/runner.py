@@ -359,14 +359,15 @@ class ModelRunner:
         return ctx, meta["new_lens"]
 
     @torch.no_grad()
-    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+    def step(self, entries: list[StepEntry], keep: bool = True) -> torch.Tensor | None:
         """Runs the batch and returns float32 logits [wanted, vocab] in the order of the
-        entries and of each entry's ``want`` (None if nothing is wanted)."""
+        entries and of each entry's ``want`` (None if nothing is wanted). With ``keep=False`` the result may be
+        memory that the next step overwrites (a caller that samples at once saves the copy)."""
         if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)
                 and not self.state_pools):
             bucket = next(b for b in self.graph_buckets if b >= len(entries))
             if self._graphs.get(bucket, ...) is not None:
-                return self._graph_step(entries, bucket)
+                return self._graph_step(entries, bucket, keep)
         ctx, new_lens = self.build_context(entries)
         if self.device.type == "cuda":
             from ..native import ops
@@ -388,7 +389,7 @@ class ModelRunner:
                 view.v[pages] = float("nan")
 
     # ------------------------------------------------------------------ decode steps as HIP graphs
-    def _graph_step(self, entries: list[StepEntry], bucket: int) -> torch.Tensor | None:
+    def _graph_step(self, entries: list[StepEntry], bucket: int, keep: bool = True) -> torch.Tensor | None:
         """A step of single tokens: the batch is padded to the bucket, written into the bucket's fixed index
         buffer, and the bucket's graph (embedding to logits of every row) is replayed."""
         width = -(-self.max_model_len // self.page_size)
@@ -415,7 +416,7 @@ class ModelRunner:
         if not rows:
             return None
         if rows == list(range(len(entries))):
-            return g["logits"][:len(entries)].clone()
+            return g["logits"][:len(entries)].clone() if keep else g["logits"][:len(entries)]
         return g["logits"][torch.tensor(rows, device=self.device)]
 
     def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int) -> dict:

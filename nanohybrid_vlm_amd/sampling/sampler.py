@@ -32,15 +32,45 @@ def noise_key(seed: int, request: int, step: int) -> int:
 class Sampler:
     def __init__(self, vocab_size: int):
         self.vocab_size = vocab_size
+        self._staged = None          # on a GPU: pinned host memory and its device twin for temperatures, keys and tokens
+
+    def _stage(self, n: int, device) -> dict:
+        """Pinned host buffers and their device twins for ``n`` rows. What a step passes to the kernel and gets
+        back goes through them with copies that do not block: a copy from ordinary host memory makes the host
+        wait until the GPU has caught up, twice a step, before the kernel is even launched."""
+        st = self._staged
+        if st is None or st["rows"] < n or st["device"] != device:
+            rows = max(64, 2 * n)
+            st = self._staged = {
+                "rows": rows, "device": device,
+                "host_temps": torch.empty(rows, dtype=torch.float32, pin_memory=True),
+                "host_keys": torch.empty(rows, dtype=torch.int64, pin_memory=True),
+                "host_tokens": torch.empty(rows, dtype=torch.int32, pin_memory=True),
+                "temps": torch.empty(rows, dtype=torch.float32, device=device),
+                "keys": torch.empty(rows, dtype=torch.int64, device=device),
+                "done": torch.cuda.Event(),
+            }
+        return st
 
     def __call__(self, logits: torch.Tensor, temperatures: list[float], keys: list[int]) -> list[int]:
         """``logits``: float32 [n, vocab] on the device; one temperature and one key per row."""
         n = logits.shape[0]
         if len(temperatures) != n or len(keys) != n:
             raise ValueError(f"{n} rows of logits, {len(temperatures)} temperatures, {len(keys)} keys")
-        temps = torch.tensor(temperatures, dtype=torch.float32).to(logits.device, non_blocking=True)
-        keys_t = torch.tensor(keys, dtype=torch.int64).to(logits.device, non_blocking=True)
-        tokens = ops.sample(logits, temps, keys_t).tolist()
+        if logits.device.type == "cuda":
+            st = self._stage(n, logits.device)
+            st["host_temps"][:n] = torch.tensor(temperatures, dtype=torch.float32)
+            st["host_keys"][:n] = torch.tensor(keys, dtype=torch.int64)
+            st["temps"][:n].copy_(st["host_temps"][:n], non_blocking=True)
+            st["keys"][:n].copy_(st["host_keys"][:n], non_blocking=True)
+            st["host_tokens"][:n].copy_(ops.sample(logits, st["temps"][:n], st["keys"][:n]), non_blocking=True)
+            st["done"].record()
+            st["done"].synchronize()
+            tokens = st["host_tokens"][:n].tolist()
+        else:
+            temps = torch.tensor(temperatures, dtype=torch.float32).to(logits.device)
+            keys_t = torch.tensor(keys, dtype=torch.int64).to(logits.device)
+            tokens = ops.sample(logits, temps, keys_t).tolist()
         for t in tokens:
             if not 0 <= t < self.vocab_size:
                 raise RuntimeError("sampling met logits that are not numbers")
