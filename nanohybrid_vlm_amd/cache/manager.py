@@ -343,6 +343,17 @@ class CacheManager:
             rc.first_live[gi] = max(rc.first_live[gi], min(passed, len(table)))
         return given_back
 
+    def rewind(self, request_id, new_len: int) -> None:
+        """Takes a commit back: the tokens from ``new_len`` on count as not stored (a step that was issued ahead of
+        its turn and is run again). Pages stay reserved. Not with windows (their pages may be gone) and not with
+        shared prefixes (pages may have become known by a content that is taken back)."""
+        rc = self.requests[request_id]
+        if self.share_prefixes or any(g.window is not None for g in self.groups):
+            raise CacheError("rewind: not with windows or shared prefixes")
+        if not 0 <= new_len <= rc.num_tokens:
+            raise CacheError(f"request {request_id!r}: rewind to {new_len} from {rc.num_tokens}")
+        rc.num_tokens = new_len
+
     def release(self, request_id) -> list[list[int]]:
         """Give back everything the request holds (block_manager.py:751-802:
         pages go back in reverse order). Returns the pages given back, per group."""

@@ -24,6 +24,7 @@ class EngineConfig:
     gpu_memory_utilization: float = 0.9
     enforce_eager: bool = False                 # True: no HIP graphs for decode
     max_graph_batch: int = 64                   # decode steps of up to this many requests replay a graph
+    run_ahead: bool = True                      # a decode step that is bound to follow is issued before the host knows the tokens it feeds
     eos: int = -1                               # filled from config.json when -1
     kvcache_block_size: int = 256               # tokens in a page (any positive number)
     num_kvcache_blocks: int = -1                # -1: sized from free memory

@@ -126,6 +126,8 @@ class LLM:
         self._sequences: dict[int, Sequence] = {}
         self._metrics: dict[int, RequestMetrics] = {}
         self._completed_metrics: list[RequestMetrics] = []
+        self._ahead = None               # a decoding step issued before its tokens were known to the host (see step)
+        self.num_steps_ahead = 0         # steps that were already under way when their turn came
 
     # ------------------------------------------------------------------ requests
     def add_request(self, prompt, sampling_params: SamplingParams | None = None) -> int:
@@ -168,14 +170,37 @@ class LLM:
             m = self._metrics[seq.seq_id]
             if m.first_scheduled is None:
                 m.first_scheduled = t0
-        logits = self.runner.step(entries, keep=False)          # sampled from at once
+        ids = [e.request_id for e in entries]
+        ahead, self._ahead = self._ahead, None
+        issued = False
+        if ahead is not None:
+            if num_prefill_tokens == 0 and set(ids) <= set(ahead["requests"]):
+                # the step issued ahead is this one (a request that ended meanwhile had its row in it for nothing;
+                # one that lives on but is not planned now takes its token back)
+                self.runner.undo_ahead(ahead, set(ahead["requests"]) - set(ids))
+                logits = self.runner.logits_ahead(ahead, ids)
+                issued = True
+                self.num_steps_ahead += 1
+            else:
+                self.runner.undo_ahead(ahead, set(ahead["requests"]))       # the plan is another: as if never issued
+        if not issued:
+            logits = self.runner.step(entries, keep=False)                  # sampled from at once
         tokens_by_id = {}
         if sampled_rows:
             seed = self.config.seed
             temps = [s.temperature for s in sampled_rows]
             keys = [noise_key(seed if s.seed is None else s.seed, s.seq_id, s.num_completion_tokens)
                     for s in sampled_rows]
-            tokens = self.sampler(logits, temps, keys)
+            launched = self.sampler.launch(logits, temps, keys)
+            # While the host waits for the tokens, ends this step and plans the next, the GPU would wait: if the
+            # next step is bound to be these requests' next tokens (nothing waits, nobody reaches max_tokens; only
+            # an end-of-sequence token can still end one), it is issued now, fed from the tokens on the device.
+            if (self.config.run_ahead and num_prefill_tokens == 0 and len(sampled_rows) == len(seqs)
+                    and not self.scheduler.waiting
+                    and all(s.num_completion_tokens + 1 < s.max_tokens for s in seqs)
+                    and self.runner.can_step_ahead(ids)):
+                self._ahead = self.runner.step_ahead(ids, launched["tokens"])
+            tokens = self.sampler.finish(launched)
             tokens_by_id = {s.seq_id: t for s, t in zip(sampled_rows, tokens)}
         finished = self.scheduler.postprocess(seqs, [tokens_by_id.get(s.seq_id) for s in seqs])
         now = perf_counter()

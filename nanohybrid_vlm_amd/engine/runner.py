@@ -419,6 +419,59 @@ class ModelRunner:
             return g["logits"][:len(entries)].clone() if keep else g["logits"][:len(entries)]
         return g["logits"][torch.tensor(rows, device=self.device)]
 
+    # ------------------------------------------------------------------ a decoding step issued ahead of its tokens
+    def can_step_ahead(self, request_ids: list) -> bool:
+        """Whether the next tokens of these requests can be run before the host knows them (``step_ahead``):
+        a recorded graph for their number, laid out for their lengths, and a cache whose commits can be taken back."""
+        if not (self.use_graphs and request_ids and len(request_ids) <= self.max_graph_batch and not self.state_pools
+                and not self.cache.share_prefixes and all(g.window is None for g in self.cache.groups)):
+            return False
+        g = self._graphs.get(next(b for b in self.graph_buckets if b >= len(request_ids)))
+        if g is None or g["graph"] is None:
+            return False
+        longest = max(256, max(self.cache.num_tokens(r) for r in request_ids) + 1)
+        need = [0] * len(self.cache.groups)
+        for r in request_ids:
+            for gi, n in enumerate(self.cache.pages_needed(r, self.cache.num_tokens(r) + 1)):
+                need[gi] += n
+        return (g["planned"] // 2 < longest <= g["planned"] + g["planned"] // 2 and longest <= self.max_model_len
+                and longest <= self.max_position and all(n <= self.cache.num_free_pages(gi) for gi, n in enumerate(need)))
+
+    @torch.no_grad()
+    def step_ahead(self, request_ids: list, tokens: torch.Tensor) -> dict:
+        """Issues the decoding step that feeds ``tokens[i]`` (int32, on the device: what the sampling kernel has
+        just been asked for, not yet known to the host) to ``request_ids[i]``, by the graph of that size; only after
+        ``can_step_ahead``. The GPU goes from one step into the next while the host still waits for the tokens,
+        finishes the step before and plans: between two steps that the host issues in turn the GPU waits 0.1 to
+        0.3 ms. Returns what ``logits_ahead`` and ``undo_ahead`` need."""
+        entries = [StepEntry(r, [0], [0]) for r in request_ids]
+        bucket = next(b for b in self.graph_buckets if b >= len(entries))
+        g = self._graphs[bucket]
+        width = -(-self.max_model_len // self.page_size)
+        arrays, meta = self._layout(entries, pad_to=bucket, table_width=width)
+        g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
+        self._copy_issued()
+        g["index"][:len(entries)].copy_(tokens[:len(entries)])     # the token ids are the first of the index arrays
+        g["graph"].replay()
+        for e, n in zip(entries, meta["new_lens"]):
+            self.cache.commit(e.request_id, n)
+        return {"requests": list(request_ids), "starts": meta["starts"], "logits": g["logits"]}
+
+    def logits_ahead(self, ahead: dict, request_ids: list) -> torch.Tensor:
+        """The logits of ``request_ids`` (some or all of the step's, in any order) from a step issued ahead."""
+        if request_ids == ahead["requests"]:
+            return ahead["logits"][:len(request_ids)]
+        place = {r: i for i, r in enumerate(ahead["requests"])}
+        return ahead["logits"][torch.tensor([place[r] for r in request_ids], device=self.device)]
+
+    def undo_ahead(self, ahead: dict, request_ids: list) -> None:
+        """Takes a step issued ahead back for these of its requests, as far as they still hold anything: their
+        tokens count as not fed (the keys and values it stored are stored again, the same, when the step is run
+        in its turn)."""
+        for r, start in zip(ahead["requests"], ahead["starts"]):
+            if r in request_ids and r in self.cache and self.cache.num_tokens(r) == start + 1:
+                self.cache.rewind(r, start)
+
     def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int) -> dict:
         """Runs the bucket's step once eagerly on its fixed buffers (so that every kernel library is loaded
         and the allocator is warm), then records it, and checks the graph if a library call went into it."""

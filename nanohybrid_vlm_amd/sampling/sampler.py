@@ -54,23 +54,35 @@ class Sampler:
 
     def __call__(self, logits: torch.Tensor, temperatures: list[float], keys: list[int]) -> list[int]:
         """``logits``: float32 [n, vocab] on the device; one temperature and one key per row."""
+        return self.finish(self.launch(logits, temperatures, keys))
+
+    def launch(self, logits: torch.Tensor, temperatures: list[float], keys: list[int]) -> dict:
+        """Asks for the tokens without waiting for them; ``finish`` waits. ``["tokens"]`` of the result is the
+        int32 tensor on the device that will hold them (a caller may feed it to the next step meanwhile)."""
         n = logits.shape[0]
         if len(temperatures) != n or len(keys) != n:
             raise ValueError(f"{n} rows of logits, {len(temperatures)} temperatures, {len(keys)} keys")
-        if logits.device.type == "cuda":
-            st = self._stage(n, logits.device)
-            st["host_temps"][:n] = torch.tensor(temperatures, dtype=torch.float32)
-            st["host_keys"][:n] = torch.tensor(keys, dtype=torch.int64)
-            st["temps"][:n].copy_(st["host_temps"][:n], non_blocking=True)
-            st["keys"][:n].copy_(st["host_keys"][:n], non_blocking=True)
-            st["host_tokens"][:n].copy_(ops.sample(logits, st["temps"][:n], st["keys"][:n]), non_blocking=True)
-            st["done"].record()
-            st["done"].synchronize()
-            tokens = st["host_tokens"][:n].tolist()
-        else:
+        if logits.device.type != "cuda":
             temps = torch.tensor(temperatures, dtype=torch.float32).to(logits.device)
             keys_t = torch.tensor(keys, dtype=torch.int64).to(logits.device)
-            tokens = ops.sample(logits, temps, keys_t).tolist()
+            return {"n": n, "tokens": ops.sample(logits, temps, keys_t), "staged": None}
+        st = self._stage(n, logits.device)
+        st["host_temps"][:n] = torch.tensor(temperatures, dtype=torch.float32)
+        st["host_keys"][:n] = torch.tensor(keys, dtype=torch.int64)
+        st["temps"][:n].copy_(st["host_temps"][:n], non_blocking=True)
+        st["keys"][:n].copy_(st["host_keys"][:n], non_blocking=True)
+        tokens = ops.sample(logits, st["temps"][:n], st["keys"][:n])
+        st["host_tokens"][:n].copy_(tokens, non_blocking=True)
+        st["done"].record()
+        return {"n": n, "tokens": tokens, "staged": st}
+
+    def finish(self, launched: dict) -> list[int]:
+        st, n = launched["staged"], launched["n"]
+        if st is None:
+            tokens = launched["tokens"].tolist()
+        else:
+            st["done"].synchronize()
+            tokens = st["host_tokens"][:n].tolist()
         for t in tokens:
             if not 0 <= t < self.vocab_size:
                 raise RuntimeError("sampling met logits that are not numbers")

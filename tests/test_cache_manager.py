@@ -271,3 +271,22 @@ def test_random_orders_with_shared_pages(seed):
         m.release(rid)
     m.check()
     assert m.num_free_pages() == 20 and m.num_shared_tokens > 0
+
+
+def test_a_commit_can_be_taken_back():
+    m = make(pages=8, page=4)
+    m.admit("a")
+    m.reserve("a", 6)
+    m.commit("a", 5)
+    m.reserve("a", 6)
+    m.commit("a", 6)
+    m.rewind("a", 5)                                        # the step that stored token 5 counts as not issued
+    assert m.num_tokens("a") == 5 and len(m.block_table("a")) == 2
+    m.commit("a", 6)
+    with pytest.raises(CacheError):
+        m.rewind("a", 7)
+    m.check()
+    with pytest.raises(CacheError):                         # a window's pages may be gone
+        w = make(pages=6, page=4, window=6)
+        w.admit("a"); w.reserve("a", 4); w.commit("a", 4)
+        w.rewind("a", 3)

@@ -177,3 +177,44 @@ def test_entry_point_refusals(model_folders, emulated_kernels):
         SamplingParams(temperature=-1)
     with pytest.raises(ValueError):
         SamplingParams(temperature=float("nan"))
+
+
+@pytest.mark.gpu
+def test_steps_issued_ahead_change_no_token(model_folders):
+    """A decoding step that is bound to follow is issued before the host knows the tokens it feeds (they go from
+    the sampling kernel to the next step on the device). Whatever ends a request meanwhile (an end-of-sequence
+    token, its max_tokens), whoever arrives late, and however few pages there are: the tokens are those of the
+    plain implementation, with steps issued ahead and without."""
+    folder = model_folders["B"]
+    cfg, w = plain.read_model_folder(folder)
+    V = cfg["vocab_size"]
+    prompts = [random_tokens(V, n, 90 + n) for n in (3, 9, 20, 31, 40, 2)]
+    greedy = SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True)
+    # an end-of-sequence token that greedy decoding of the first prompt meets on its way
+    eos = _plain_generate(cfg, w, prompts[0], greedy, 0, 0, None)[6]
+    params = [SamplingParams(temperature=0.0, max_tokens=24), SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True),
+              SamplingParams(temperature=0.9, max_tokens=20, seed=5), SamplingParams(temperature=0.0, max_tokens=1),
+              SamplingParams(temperature=0.0, max_tokens=2), SamplingParams(temperature=0.7, max_tokens=17)]
+    want = [_plain_generate(cfg, w, p, sp, i, 0, eos) for i, (p, sp) in enumerate(zip(prompts, params))]
+    assert len(want[0]) < 24, "the first request was meant to end at the end-of-sequence token"
+    for pages in (64, 14):                                  # ample, and so few that requests are pushed out
+        ahead_steps = {}
+        for run_ahead in (False, True):
+            llm = LLM(folder, dtype="float32", kvcache_block_size=8, num_kvcache_blocks=pages, max_num_batched_tokens=16,
+                      eos=eos, run_ahead=run_ahead)
+            done = {}
+            for p, sp in zip(prompts[:3], params[:3]):
+                llm.add_request(p, sp)
+            for _ in range(9):                              # the others arrive while the first three decode
+                done.update(llm.step()[0])
+            for p, sp in zip(prompts[3:], params[3:]):
+                llm.add_request(p, sp)
+            while not llm.is_finished():
+                done.update(llm.step()[0])
+            assert [done[i] for i in range(len(prompts))] == want, f"run_ahead={run_ahead}, {pages} pages"
+            llm.runner.cache.check()
+            assert llm.get_memory_stats()["groups"][0]["free_pages"] == pages
+            ahead_steps[run_ahead] = llm.num_steps_ahead
+            if pages == 14:
+                assert llm.scheduler.num_preemptions > 0, "the small cache was meant to force a request out"
+        assert ahead_steps[False] == 0 and ahead_steps[True] >= 10
