@@ -187,10 +187,12 @@ class NativeBackend:
         if window:
             span = min(span, window + 64)
         # about a thousand waves, one per SIMD of the chip, was the fastest at every batch size measured
-        # (2,176 keys, 1 to 64 requests); too long a split costs more than too short a one, so round down
+        # (2,176 keys, 1 to 64 requests); too long a split costs more than too short a one, so round down,
+        # and no split is longer than 512 keys (64 requests: 110 us with splits of 512, 117 us with 1,024,
+        # 161 us with 2,048; a wave takes its keys one round after the other)
         want = max(1, T * Hkv * span // 1024)
         split_len = 64
-        while split_len * 2 <= want and split_len < 1024:
+        while split_len * 2 <= want and split_len < 512:
             split_len *= 2
         n_splits = -(-batch.max_context_len // split_len)
         part_o = torch.empty((T, Hq, n_splits, D), dtype=torch.float32, device=q.device)
