@@ -186,13 +186,15 @@ class NativeBackend:
         span = min(self.planned_context, batch.max_context_len) if self.planned_context else batch.max_context_len
         if window:
             span = min(span, window + 64)
-        # about a thousand waves, one per SIMD of the chip, was the fastest at every batch size measured
-        # (2,176 keys, 1 to 64 requests); too long a split costs more than too short a one, so round down,
-        # and no split is longer than 512 keys (64 requests: 110 us with splits of 512, 117 us with 1,024,
-        # 161 us with 2,048; a wave takes its keys one round after the other)
+        # One wave per SIMD of the chip (about a thousand) is the fastest while that leaves splits of up to 256
+        # keys, half as many waves again from there on (a wave takes its keys one round after the other), and no
+        # split is longer than 1,024 keys. Measured at 2,176 and 8,192 keys, 1 to 64 requests, 8 key/value heads: the
+        # best split length is 64 to 128 keys for 8 x 2,176 keys in all, 256 for 32 x 2,176 (62 against 64 us with
+        # 512), 512 for 48 and 64 x 2,176 (110 against 118 us with 1,024) and for 16 x 8,192, 1,024 for 32 x 8,192.
         want = max(1, T * Hkv * span // 1024)
+        want = min(want, max(256, want * 2 // 3))
         split_len = 64
-        while split_len * 2 <= want and split_len < 512:
+        while split_len * 2 <= want and split_len < 1024:
             split_len *= 2
         n_splits = -(-batch.max_context_len // split_len)
         part_o = torch.empty((T, Hq, n_splits, D), dtype=torch.float32, device=q.device)
