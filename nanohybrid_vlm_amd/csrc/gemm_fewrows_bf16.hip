@@ -126,8 +126,9 @@ typedef const __attribute__((address_space(1))) void* global_ptr;
 // The kernel with x resident in LDS: x_s[m][K + 8] (the 16 bytes between rows spread the rows over the
 // banks), then for tile = blockIdx.x, + gridDim.x, ...: waves split K as above, sums meet in one of two
 // LDS buffers (one barrier a tile), and the waves take turns in adding them up and writing the result.
-// (Asking for the next tile's first loads before a tile's sums are exchanged was measured and changed nothing;
-// asking for the first tile's first weights before x made every shape slower, by 0.5 to 3 us.)
+// The first weights of a block's first tile are asked for right after x and the wait before the first product is for
+// x alone (0.2 to 0.5 us less per call at every shape; asked for before x they made every shape slower, by 0.5 to
+// 3 us). (Asking for the next tile's first loads before a tile's sums are exchanged was measured and changed nothing.)
 template <int WAVES, int UNROLL, bool GLU, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                            const bf16_t* __restrict__ bias, TOut* __restrict__ y,
@@ -148,12 +149,28 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
     if (piece < pieces_per_row)
       __builtin_amdgcn_global_load_lds((global_ptr)(x + (size_t)m * K + piece * 8), (lds_ptr)(x_s + m * pitch + part * 512), 16, 0, 0);
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
   const int ksteps = (K + 31) / 32;
   const int first = wave * steps_per_wave;
   const int last = min(first + steps_per_wave, ksteps);
+  // The first weights of the block's first tile are asked for while x is still on its way: every lane asks (from an
+  // address moved into the matrix where it would lie outside), so that exactly UNROLL NA loads are younger than
+  // those of x, and the wait below is for x alone.
+  asm volatile("" ::: "memory");
+  bf16x8 a_first[UNROLL][NA];
+  {
+    const int n0 = blockIdx.x * 16;
+    const bool n_ok = n0 + col < N;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int k = (first + u) * 32 + grp * 8;
+      const int k_in = k + 8 <= K ? k : 0;
+#pragma unroll
+      for (int na = 0; na < NA; ++na) a_first[u][na] = load8(w + ((size_t)na * N + (n_ok ? n0 + col : 0)) * K + k_in);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(UNROLL * NA) : "memory");
+  __syncthreads();
+
   const bool m_ok = col < M;
   const bf16_t* xrow_s = x_s + (m_ok ? col : 0) * pitch;
   int parity = 0, turn = 0;
@@ -168,12 +185,16 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
     for (int na = 0; na < NA; ++na) acc[na] = floatx4{0.f, 0.f, 0.f, 0.f};
     for (int s0 = first; s0 < last; s0 += UNROLL) {
       bf16x8 a[UNROLL][NA];
+      const bool asked = tile == (int)blockIdx.x && s0 == first;
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const int k = (s0 + u) * 32 + grp * 8;
         const bool k_ok = (s0 + u < last) && k < K;
 #pragma unroll
-        for (int na = 0; na < NA; ++na) a[u][na] = (n_ok && k_ok) ? load8(wrow[na] + k) : zero8();
+        for (int na = 0; na < NA; ++na) {
+          if (asked) a[u][na] = (n_ok && k_ok) ? a_first[u][na] : zero8();
+          else a[u][na] = (n_ok && k_ok) ? load8(wrow[na] + k) : zero8();
+        }
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
