@@ -24,7 +24,12 @@
 // microseconds saved at 8 requests and lost time at 1 and at 64. So were rounds of 64 keys for launches of one
 // wave per SIMD (5 % less time at 1 and 2 requests, more at 4 and above), and values loaded straight into LDS
 // (global_load_lds, read with ds_read_b64_tr_b16 as in the prompt kernel) with the next round's keys and values
-// asked for before this round is computed: 3 to 8 % less time for this kernel, 1 % of a decoding step.)
+// asked for before this round is computed: 3 to 8 % less time for this kernel, 1 % of a decoding step. And blocks of two
+// or four waves that take a split's rounds in turn and meet in wave 0 at the end, lane by lane, so that longer splits
+// leave fewer partial results to write and to merge for the same number of waves at work: alone, over caches that
+// change from call to call, 10 % less time at 16 and 32 requests of 2,176 keys (four waves on splits of 512 against one
+// wave on splits of 256), nothing at 1, 8 and 64 requests or at 8,192 keys; inside the model's decoding step the same
+// choice took 2 to 5 % more time at 24, 32 and 48 requests.)
 #include "nhv_common.h"
 #include <math.h>
 
