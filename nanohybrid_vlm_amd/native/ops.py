@@ -255,7 +255,8 @@ class NativeBackend:
         Which is fastest depends on the shape in ways no rule here captures, and the library's own first guess is
         often far from its best (a 5120 x 17408 weight against 8 rows: 112 us by its first guess, 37 us by another
         of its algorithms, 50 us by the own kernel; a 4096 x 12288 weight: 22, 22 and 25 us; the same weight
-        against 2,048 rows: 197 us by ``torch.mm``, 173 us by the library's second guess). So a shape is timed in
+        against 128 rows: 67 us by ``torch.mm``, 43 us by the library's sixth guess; against 2,048 rows the first
+        guess is as good as any). So a shape is timed in
         every way there is, once, and the answer is kept for the life of the process: a shape of up to
         ``library_rows`` rows while ``measure_linears`` is set (the run before a graph is recorded), a shape of
         more rows (a portion of a prompt) in the third step that meets it, since only the sizes that come again
