@@ -529,3 +529,26 @@ def test_a_shape_of_many_rows_is_measured_in_the_third_step_that_meets_it(ops):
             backend.chosen[key] = saved[0]
         if saved[1] is not None:
             backend._met[key] = saved[1]
+
+
+def test_library_products_refuse_what_they_cannot_do(ops):
+    """The wrapper of the vendor's matrix library names what is wrong: an algorithm the plan does not have, a
+    workspace smaller than the plan's, a plan that was never made."""
+    import ctypes
+    from nanohybrid_vlm_amd.native.ops import KernelError
+    backend = ops.backend()
+    plan, count = backend._library_plan(8, 256, 512, False)
+    assert count > 0 and backend._library_plan(8, 256, 512, False) == (plan, count)      # a shape has one plan
+    x = rnd(8, 512, dtype=torch.bfloat16, seed=71)
+    w = rnd(256, 512, dtype=torch.bfloat16, seed=72)
+    out = torch.empty(8, 256, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(KernelError, match="algorithms"):
+        backend._library_product(x, w, out, count)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    with pytest.raises(KernelError, match="no plan"):
+        backend._call("nhv_library_gemm", 10 ** 6, 0, ptr(x), ptr(w), ptr(out), None, ctypes.c_size_t(0), None, lib=backend.blas_lib())
+    with pytest.raises(KernelError, match="result type"):
+        backend._call("nhv_library_gemm_plan", 8, 256, 512, 7, 4, ctypes.c_size_t(0), ctypes.byref(ctypes.c_int()),
+                      ctypes.byref(ctypes.c_int()), lib=backend.blas_lib())
+    backend._library_product(x, w, out, 0)
+    torch.testing.assert_close(out.double(), x.double() @ w.double().T, **tol(torch.bfloat16))
