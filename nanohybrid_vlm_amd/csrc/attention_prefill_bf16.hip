@@ -8,8 +8,8 @@
 // first: with 4 heads per key/value head a block is 16 or 32 tokens x 4 heads, and every
 // key and value it stages in LDS is used by 64 or 128 rows. With two row tiles a wave
 // reads every operand of keys and values from LDS once for both (the reads from LDS are
-// what the kernel waits for most); that is taken where the batch still fills the chip
-// with blocks of that size. Keys are taken in tiles of 64, in rising order:
+// what the kernel waits for most); that is taken where the batch still gives every
+// compute unit two blocks of that size. Keys are taken in tiles of 64, in rising order:
 //   S^T[key, row] = K[key, :] . Q[row, :]      K tile from LDS, Q in registers (v_mfma_f32_16x16x32_bf16)
 //   running maximum per row in float (two shuffles over the lane groups), sums kept per lane
 //   O^T[d, row]  += V^T[d, key] . P^T[key, row]  V^T from LDS, P in registers (v_mfma_f32_16x16x32_bf16)
@@ -372,8 +372,9 @@ extern "C" int nhv_prefill_attention_bf16(const void* q, const void* k_cache, co
     if (page_size == (1 << b)) page_shift = b;
   const int G = Hq / Hkv;
   const long long row_tiles = (long long)G * ((max_q_len + 15) / 16);
-  // two row tiles a wave where that still leaves a block for every compute unit
-  const bool two = prefill::MAX_RT >= 2 && (row_tiles + 7) / 8 * Hkv * B >= 256;
+  // two row tiles a wave where that still leaves two blocks for every compute unit (1,024 new tokens of 8 kv heads
+  // are 256 such blocks: 41 us, and 31 us as 512 blocks of one row tile a wave; after 7,000 keys 259 and 216 us)
+  const bool two = prefill::MAX_RT >= 2 && (row_tiles + 7) / 8 * Hkv * B >= 512;
   const int tpb = two ? 8 : 4;
   const long long gx = (row_tiles + tpb - 1) / tpb;
   NHV_REQUIRE(gx <= 0x7fffffff && Hkv <= 65535 && B <= 65535, "prefill attention: grid too large");
