@@ -284,6 +284,9 @@ class NativeBackend:
             how = self._measure(x, w, out, gated, many)
         except torch.OutOfMemoryError:
             how = RULE if many else None                     # no room to measure: the rule
+        finally:
+            if many:
+                self._sweep = None                           # (a step of prompt portions is followed by no end_measurements)
         if how is not None:
             self.chosen[key] = how
             if gated and how >= 0:
@@ -351,8 +354,6 @@ class NativeBackend:
                   f"{'-' if incumbent_time is None else format(1e3 * incumbent_time, '.1f')} us, library's first guess "
                   f"{1e3 * first_guess:.1f} us, fastest {1e3 * best[0][0]:.1f} us ({name.get(best[0][1], best[0][1])} "
                   f"of {len(runs)} ways); taken: {name.get(how, how)}", file=sys.stderr, flush=True)
-        if many:
-            self._sweep = None                               # (a step of prompt portions is followed by no end_measurements)
         return how
 
     def end_measurements(self) -> None:
