@@ -262,7 +262,8 @@ class NativeBackend:
         more rows (a portion of a prompt) in the third step that meets it, since only the sizes that come again
         and again (portions that fill the token budget) are worth the 50 ms. An algorithm whose result differs
         from the trusted way's (own kernel, ``torch.mm``) by more than rounding, or from its own on a second run,
-        is left out. The trusted way stays unless a library algorithm takes less than 0.95 of its time."""
+        is left out. The trusted way stays unless a library algorithm takes less than 0.95 of its time (0.90 for the
+        gated projection)."""
         M, K = x.shape
         N = w.shape[0]
         float_result = out.dtype == torch.float32
@@ -345,7 +346,9 @@ class NativeBackend:
         best = sorted((min(t, self._time_cold(runs[how], 8)), how) for t, how in finalists)
         how = best[0][1]
         incumbent_time = next((t for t, h in best + once if h == incumbent), None)
-        if incumbent_time is not None and how != incumbent and best[0][0] >= 0.95 * incumbent_time:
+        # (the fused gated kernel gives way only to a clear win: the library's way is two kernels, and the second one's
+        # cost inside a step is the harder one to measure alone)
+        if incumbent_time is not None and how != incumbent and best[0][0] >= (0.90 if gated else 0.95) * incumbent_time:
             how = incumbent
         if os.environ.get("NHV_SHOW_MEASUREMENTS"):
             name = {OWN: "own", RULE: "torch.mm"}
