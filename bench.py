@@ -40,29 +40,20 @@ def parse_args():
 
 
 def build_llm(args, max_seqs):
-    import torch
     from nanohybrid_vlm_amd import LLM
-    from nanohybrid_vlm_amd.config.registry import resolve_architecture
-    from nanohybrid_vlm_amd.parts.model import DecoderModel
-    from nanohybrid_vlm_amd.shapes import SHAPES
-    from nanohybrid_vlm_amd.weights.random_init import fill_random_on_device
+    from nanohybrid_vlm_amd.config.registry import named_shapes
 
-    raw = dict(SHAPES[args.shape])
+    raw = dict(named_shapes()[args.shape])
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
-    arch = resolve_architecture(raw)
-    cfg = arch.parse_config(raw)
-    model = DecoderModel(arch.build_spec(cfg))
-    dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
-    fill_random_on_device(model, seed=0, dtype=dtype, device="cuda:0")
     pages_per_seq = -(-args.context // args.block_size)
-    llm = LLM(f"random {args.shape}", built_model=(arch, cfg, model), dtype=args.dtype,
+    llm = LLM(raw, random_weights=0, dtype=args.dtype,
               kvcache_block_size=args.block_size, num_kvcache_blocks=max_seqs * pages_per_seq + 1,
               max_num_seqs=max_seqs, max_num_batched_tokens=max(2048, max_seqs), max_model_len=args.context,
               scheduler_policy="prefill_first",     # while prompts are fed nothing decodes, so all requests decode in step
               enforce_eager=args.eager, **({"max_graph_batch": args.max_graph_batch} if args.max_graph_batch else {}))
-    return llm, cfg, full_layers
+    return llm, llm.runner.cfg, full_layers
 
 
 def model_bytes_and_flops(cfg, itemsize):

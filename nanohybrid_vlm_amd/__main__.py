@@ -37,9 +37,11 @@ def _case(text: str) -> tuple[int, int]:
 def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--model", help="folder with config.json and model.safetensors")
     ap.add_argument("--random-weights", type=int, metavar="SEED",
-                    help="instead of --model: random weights of --shape, drawn on the device")
-    ap.add_argument("--shape", default="tinyA", choices=("tinyA", "tinyB", "8b", "14b", "32b"),
-                    help="sizes of the model for --random-weights")
+                    help="instead of --model: random weights of --shape or --config, drawn on the device")
+    ap.add_argument("--shape", default="tinyA",
+                    help="with --random-weights: a named configuration of a registered architecture "
+                         "(Qwen3: tinyA, tinyB, 8b, 14b, 32b)")
+    ap.add_argument("--config", help="with --random-weights: a config.json to take the sizes from, instead of --shape")
     ap.add_argument("--layers", type=int, help="with --random-weights: override num_hidden_layers")
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32", "bf16", "fp32"))
     ap.add_argument("--mode", choices=("eager", "graph"), default="graph", help="graph: decode steps replay HIP graphs")
@@ -56,30 +58,42 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--enable-prefix-cache", action="store_true",
                     help="requests with a common start share the full pages that hold it")
+    ap.add_argument("--plugin", action="append", metavar="MODULE",
+                    help="a module to import first: it may register architectures and parts of its own; repeatable")
+
+
+def _import_plugins(names) -> None:
+    """Modules that register architectures or parts of their own when imported."""
+    import importlib
+    for name in names or []:
+        importlib.import_module(name)
+
+
+def _named_config(args) -> dict:
+    """config.json contents for --random-weights and random-model: a file, or a registered architecture's named shape."""
+    from .config.registry import named_shapes
+    if getattr(args, "config", None):
+        raw = json.loads(Path(args.config).read_text())
+    else:
+        shapes = named_shapes()
+        if args.shape not in shapes:
+            raise SystemExit(f"unknown --shape '{args.shape}'; known: {sorted(shapes)}")
+        raw = dict(shapes[args.shape])
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    return raw
 
 
 def _make_llm(args):
     from . import LLM
+    _import_plugins(args.plugin)
     if (args.model is None) == (args.random_weights is None):
         raise SystemExit("give either --model DIR or --random-weights SEED")
-    built, label = None, args.model
+    model, random_weights = args.model, None
     if args.random_weights is not None:
-        import torch
-        from .config.registry import resolve_architecture
-        from .parts.model import DecoderModel
-        from .shapes import SHAPES
-        from .weights.random_init import fill_random_on_device
-        raw = dict(SHAPES[args.shape])
-        if args.layers:
-            raw["num_hidden_layers"] = args.layers
-        arch = resolve_architecture(raw)
-        cfg = arch.parse_config(raw)
-        model = DecoderModel(arch.build_spec(cfg))
-        dtype = torch.bfloat16 if args.dtype in ("bfloat16", "bf16") else torch.float32
-        fill_random_on_device(model, seed=args.random_weights, dtype=dtype, device="cuda:0")
-        built, label = (arch, cfg, model), f"random {args.shape}"
-        args.model = label
-    return LLM(label, built_model=built, dtype=args.dtype, enforce_eager=args.mode == "eager",
+        model, random_weights = _named_config(args), args.random_weights
+        args.model = f"random {args.config or args.shape}"
+    return LLM(model, random_weights=random_weights, dtype=args.dtype, enforce_eager=args.mode == "eager",
                max_num_batched_tokens=args.token_budget, gpu_memory_utilization=args.gpu_memory_utilization,
                kvcache_block_size=args.block_size, num_kvcache_blocks=args.num_blocks, max_num_seqs=args.max_num_seqs,
                max_model_len=args.max_model_len, scheduler_policy=args.scheduler_policy, seed=args.seed,
@@ -181,15 +195,9 @@ def cmd_bench(args) -> int:
 
 
 def cmd_random_model(args) -> int:
-    from .shapes import SHAPES
     from .weights.random_init import write_random_model
-    if args.config:
-        raw = json.loads(Path(args.config).read_text())
-    else:
-        raw = dict(SHAPES[args.shape])
-    if args.layers:
-        raw["num_hidden_layers"] = args.layers
-    write_random_model(args.out, raw, args.seed, args.store_dtype)
+    _import_plugins(args.plugin)
+    write_random_model(args.out, _named_config(args), args.seed, args.store_dtype)
     print(args.out)
     return 0
 
@@ -235,8 +243,10 @@ def main(argv=None) -> int:
 
     r = sub.add_parser("random-model", help="write a model folder with seeded random weights")
     r.add_argument("--out", required=True)
-    r.add_argument("--shape", default="tinyA", choices=("tinyA", "tinyB", "8b", "14b", "32b"))
+    r.add_argument("--shape", default="tinyA", help="a named configuration of a registered architecture")
     r.add_argument("--config", help="a config.json to use instead of a named shape")
+    r.add_argument("--plugin", action="append", metavar="MODULE",
+                   help="a module to import first: it may register architectures and parts of its own; repeatable")
     r.add_argument("--layers", type=int, help="override num_hidden_layers")
     r.add_argument("--seed", type=int, default=0)
     r.add_argument("--store-dtype", default="bfloat16", choices=("bfloat16", "float32"))

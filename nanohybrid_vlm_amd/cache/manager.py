@@ -186,6 +186,9 @@ class CacheManager:
     def num_free_pages(self, group: int = 0) -> int:
         return self.pools[group].num_free
 
+    def num_free_slots(self) -> int:
+        return len(self.slots.free)
+
     def pages_needed(self, request_id, new_len: int) -> list[int]:
         """Pages that ``reserve(request_id, new_len)`` would take, per group.
         ``request_id`` may be unknown (a request not yet admitted)."""

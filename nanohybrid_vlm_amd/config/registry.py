@@ -9,7 +9,7 @@ parts of every layer and the run order) and the names of the checkpoint's tensor
 from __future__ import annotations
 
 import importlib
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Callable
 
 
@@ -25,6 +25,9 @@ class WeightSource:
     param: str
     row_start: int = 0
     rows: int | None = None        # None: the whole parameter
+    # a second copy of what another checkpoint tensor already gives the same parameter (a tied head stored beside
+    # the embedding): the file may leave it out; if it is there it must hold the same numbers as the first
+    copy: bool = False
 
 
 @dataclass(frozen=True)
@@ -34,8 +37,8 @@ class Architecture:
     parse_config: Callable                      # raw dict -> typed configuration
     build_spec: Callable                        # typed configuration -> ModelSpec
     checkpoint_names: Callable                  # typed configuration -> {checkpoint tensor name: WeightSource}
-    optional_names: Callable = lambda cfg: set()  # checkpoint names that may be absent or present
     ignored_prefixes: tuple[str, ...] = ()      # checkpoint names under these are skipped (nanovllm/utils/loader.py:27-31)
+    named_shapes: dict = field(default_factory=dict)   # name -> config.json contents, for measurements and examples
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}
@@ -64,6 +67,16 @@ def _get(name: str) -> Architecture | None:
 
 def registered_architectures() -> list[str]:
     return sorted(set(_ARCHITECTURES) | set(_LAZY))
+
+
+def named_shapes() -> dict[str, dict]:
+    """Every registered architecture's named configurations (config.json contents by name)."""
+    out: dict[str, dict] = {}
+    for name in registered_architectures():
+        arch = _get(name)
+        if arch is not None:
+            out.update(arch.named_shapes)
+    return out
 
 
 def resolve_architecture(raw_config: dict) -> Architecture:

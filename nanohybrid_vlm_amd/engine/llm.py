@@ -73,16 +73,17 @@ class RequestMetrics:
 
 
 def validate_token_ids(token_ids) -> None:
-    """A non-empty list of non-negative integers (nanovllm/inputs.py:29-55)."""
+    """A prompt of token ids is a list with at least one entry, every entry a plain integer that is not
+    negative (the reference checks the same four things, nanovllm/inputs.py:29-55)."""
     if not isinstance(token_ids, list):
-        raise TypeError("token_ids must be a list")
-    if not token_ids:
-        raise ValueError("token_ids must not be empty")
-    for t in token_ids:
-        if not isinstance(t, int) or isinstance(t, bool):
-            raise TypeError("Every token ID must be an integer")
+        raise TypeError(f"a prompt of token ids is a list, not {type(token_ids).__name__}")
+    if len(token_ids) == 0:
+        raise ValueError("a prompt needs at least one token")
+    for place, t in enumerate(token_ids):
+        if isinstance(t, bool) or not isinstance(t, int):
+            raise TypeError(f"token {place} of the prompt is {t!r}: token ids are integers")
         if t < 0:
-            raise ValueError("Token IDs must be non-negative")
+            raise ValueError(f"token {place} of the prompt is {t}: token ids are not negative")
 
 
 def _load_tokenizer(folder: str):
@@ -94,13 +95,26 @@ def _load_tokenizer(folder: str):
 
 
 class LLM:
-    def __init__(self, model: str, *, built_model=None, **kwargs):
-        """``model``: folder with config.json, model.safetensors (and tokenizer.json for text prompts).
-        ``built_model``: (architecture, typed configuration, model with weights bound) made elsewhere, e.g.
-        with random weights drawn on the device; ``model`` is then only a label."""
+    def __init__(self, model, *, random_weights: int | None = None, built_model=None, **kwargs):
+        """``model``: folder with config.json, model.safetensors (and tokenizer.json for text prompts); or the
+        contents of a config.json as a dict, together with ``random_weights=seed``: a model of that
+        configuration with random weights drawn on the device.
+        ``built_model``: (architecture, typed configuration, model with weights bound) made elsewhere;
+        ``model`` is then only a label."""
         unknown = set(kwargs) - EngineConfig.field_names()
         if unknown:
             raise TypeError(f"unknown engine options: {sorted(unknown)}; known: {sorted(EngineConfig.field_names())}")
+        if isinstance(model, dict):
+            if built_model is not None:
+                raise TypeError("give either a configuration with random_weights or built_model, not both")
+            if random_weights is None:
+                raise TypeError("a configuration in place of a model folder needs random_weights=SEED")
+            from ..weights.random_init import build_random_model
+            check = EngineConfig(model="random weights", **kwargs)           # (the options are checked before the weights are drawn)
+            built_model = build_random_model(model, random_weights, check.dtype, check.device)
+            model = f"random weights ({built_model[0].name}, seed {random_weights})"
+        elif random_weights is not None:
+            raise TypeError("random_weights goes with a configuration (a dict), not with a model folder")
         self.config = cfg = EngineConfig(model=model, **kwargs)
         if built_model is None and not os.path.isdir(model):
             raise FileNotFoundError(f"model folder '{model}' does not exist")
@@ -112,12 +126,12 @@ class LLM:
             gpu_memory_utilization=cfg.gpu_memory_utilization, max_num_batched_tokens=cfg.max_num_batched_tokens,
             model=built, arch=arch, cfg=typed, use_graphs=not cfg.enforce_eager, max_model_len=cfg.max_model_len,
             share_prefixes=cfg.enable_prefix_cache, max_graph_batch=cfg.max_graph_batch)
-        model_cfg = self.runner.cfg
         cfg.num_kvcache_blocks = self.runner.num_pages
-        # max_model_len is capped by the model's positions (nanovllm/config.py:420-423)
-        cfg.max_model_len = min(cfg.max_model_len, model_cfg.max_position_embeddings)
-        if cfg.eos == -1 and getattr(model_cfg, "eos_token_id", None) is not None:
-            cfg.eos = model_cfg.eos_token_id
+        # max_model_len is capped by the model's positions (nanovllm/config.py:420-423); both, and the token that
+        # ends a request, are facts of the built model (no field of an architecture's configuration is read here)
+        cfg.max_model_len = min(cfg.max_model_len, self.runner.max_position)
+        if cfg.eos == -1 and self.runner.eos_token_id is not None:
+            cfg.eos = self.runner.eos_token_id
         self.tokenizer = _load_tokenizer(model) if built_model is None else None
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.eos,
                                    cfg.max_model_len, cfg.scheduler_policy, cfg.max_prefill_wait_ms)

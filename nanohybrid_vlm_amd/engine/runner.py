@@ -22,7 +22,7 @@ from typing import Hashable
 import numpy as np
 import torch
 
-from ..cache.manager import NO_PAGE, CacheManager, PagedGroupSpec
+from ..cache.manager import NO_PAGE, CacheManager, OutOfPages, PagedGroupSpec
 from ..config.model_config import read_config_json
 from ..config.registry import resolve_architecture
 from ..native.ops import AttentionBatch
@@ -63,14 +63,18 @@ class ModelRunner:
             load_weights(model, arch, cfg, model_dir, self.dtype, self.device)
         self.arch, self.cfg, self.model = arch, cfg, model
         self.model.to(self.device)
+        # what the engine above needs to know of the model comes from the model's description, not from the
+        # architecture's typed configuration (whose fields are the architecture's own affair)
         self.vocab_size = model.spec.vocab_size
         self.max_position = model.spec.max_position
+        self.eos_token_id = model.spec.eos_token_id
         self.page_size = page_size
         if share_prefixes and poison_freed_pages:
             raise ValueError("a freed page keeps its content for later requests when prefixes are shared; "
                              "poison_freed_pages would destroy it")
         self.share_prefixes = share_prefixes
-        self._make_cache(page_size, num_pages, num_state_slots, gpu_memory_utilization, max_num_batched_tokens)
+        self._make_cache(page_size, num_pages, num_state_slots, gpu_memory_utilization, max_num_batched_tokens,
+                         graph_rows=max_graph_batch if use_graphs else 0)
         self._pinned = None
         self._pinned_free = None
         # a debugging aid: pages that are given back are filled with NaN, so that a read of a page that a
@@ -83,18 +87,17 @@ class ModelRunner:
         # requests is bound by its launches (8.3 ms at every size). A graph with a library call in it is checked
         # when it is recorded: replayed three times, with eager work and waits between, and compared bit by bit
         # with the eager result; a bucket whose graph fails runs eagerly from then on.
-        self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and self.model.recordable()
         self.max_model_len = min(max_model_len or self.max_position, self.max_position)
         self.max_graph_batch = max_graph_batch
-        # batch sizes that have a graph: a step is padded to the next one (powers of two and the sizes half way between)
-        sizes = sorted({b for p in range(24) for b in (1 << p, 3 << p >> 1) if b >= 1})
-        self.graph_buckets = [b for b in sizes if b < max_graph_batch] + [max_graph_batch]
+        # batch sizes that have a graph: a step is padded to the next one
+        self.graph_buckets = self._bucket_sizes(max_graph_batch)
         self._graphs: dict[int, dict | None] = {}     # None: the bucket's graph failed its check
         self.graph_check = torch.equal                # (replay, eager) -> bool; a test replaces it to force a refusal
         self.graphs_rerecorded = 0                    # graphs recorded again because the contexts had outgrown their layout
 
     # ------------------------------------------------------------------ cache
-    def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens):
+    def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens, graph_rows=0):
         needs = self.model.cache_needs()
         windows: list[int | None] = []                 # one group per distinct window
         entry_group: dict[int, int] = {}
@@ -105,35 +108,42 @@ class ModelRunner:
                 entry_group[i] = windows.index(need.window)
         if not windows:
             windows = [None]                           # a model without paged layers still has one (empty) group
-        item = torch.empty((), dtype=self.dtype).element_size()
-        page_bytes = sum(2 * page_size * n.num_kv_heads * n.head_dim * item
-                         for n in needs if isinstance(n, PagedKVNeed))
-        if num_pages is None:
-            num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens)
-        self.num_pages = num_pages
-        groups = [PagedGroupSpec(name="all keys" if w is None else f"window {w}", page_size=page_size,
-                                 num_pages=num_pages, window=w) for w in windows]
         if self.share_prefixes and any(isinstance(n, StateNeed) for n in needs):
             # state of fixed size summarises all earlier tokens: pages alone do not bring a prefix back
             # (the reference switches the page hashes off for such models, nanovllm/config.py:384-399)
             raise ValueError("prefixes cannot be shared by a model with per-request state")
-        self.cache = CacheManager(groups, num_state_slots, share_prefixes=self.share_prefixes)
         views: list[CacheView | None] = [None] * len(needs)
-        self.kv_tensors: list[torch.Tensor] = []
+        # the pools of per-request state come first, so that the pages are counted from what is left
+        # (the reference splits its budget between the two, nanovllm/engine/model_runner.py:723-775).
+        # One row more than there are slots: the padding rows of a recorded step work on it.
         self.state_pools: list[dict] = []
+        self.num_state_slots = num_state_slots
         for i, need in enumerate(needs):
-            if isinstance(need, PagedKVNeed):
-                # [2, pages, page_size, kv_heads, head_dim]: one token's heads lie together
-                # (nanovllm/engine/model_runner.py:870-906)
-                kv = torch.empty((2, num_pages, page_size, need.num_kv_heads, need.head_dim),
-                                 dtype=self.dtype, device=self.device)
-                self.kv_tensors.append(kv)
-                views[i] = CacheView(kind="paged", group=entry_group[i], k=kv[0], v=kv[1], writes=True)
-            elif isinstance(need, StateNeed):
-                pool = {name: torch.zeros((num_state_slots, *shape), dtype=dt, device=self.device)
+            if isinstance(need, StateNeed):
+                pool = {name: torch.zeros((num_state_slots + 1, *shape), dtype=dt, device=self.device)
                         for name, (shape, dt) in need.tensors.items()}
                 self.state_pools.append(pool)
                 views[i] = CacheView(kind="state", state=pool)
+        item = torch.empty((), dtype=self.dtype).element_size()
+        page_bytes = sum(2 * page_size * n.num_kv_heads * n.head_dim * item
+                         for n in needs if isinstance(n, PagedKVNeed))
+        if num_pages is None:
+            num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens, graph_rows)
+        self.num_pages = num_pages
+        groups = [PagedGroupSpec(name="all keys" if w is None else f"window {w}", page_size=page_size,
+                                 num_pages=num_pages, window=w) for w in windows]
+        self.cache = CacheManager(groups, num_state_slots, share_prefixes=self.share_prefixes)
+        self.kv_tensors: list[torch.Tensor] = []       # the pages that requests may hold, per cache unit
+        for i, need in enumerate(needs):
+            if isinstance(need, PagedKVNeed):
+                # [2, pages + 1, page_size, kv_heads, head_dim]: one token's heads lie together
+                # (nanovllm/engine/model_runner.py:870-906). The last page is handed to no request and holds zeros:
+                # the padding rows of a recorded step read their one key there.
+                kv = torch.empty((2, num_pages + 1, page_size, need.num_kv_heads, need.head_dim),
+                                 dtype=self.dtype, device=self.device)
+                kv[:, num_pages].zero_()
+                self.kv_tensors.append(kv[:, :num_pages])
+                views[i] = CacheView(kind="paged", group=entry_group[i], k=kv[0], v=kv[1], writes=True)
         for i, e in enumerate(self.model.run_order):
             if e.cache is not None:
                 lender = views[e.cache]
@@ -143,10 +153,11 @@ class ModelRunner:
                 views[i] = CacheView(kind="none")
         self.model.attach_cache(views)
 
-    def _pages_from_free_memory(self, page_bytes, utilization, max_tokens) -> int:
-        """budget = total * utilization - used - room for a step's activations
-        (nanovllm/engine/model_runner.py:654-699,839-861; the reference measures the
-        room with a warm-up pass, here it is computed from the layer sizes)."""
+    def _pages_from_free_memory(self, page_bytes, utilization, max_tokens, graph_rows) -> int:
+        """budget = total * utilization - used - room for a step's activations - room for the recorded steps
+        (nanovllm/engine/model_runner.py:654-699,839-861; the reference measures the room with a warm-up pass,
+        here it is computed from the layer sizes). The weights and the state pools are allocated already and
+        count as used."""
         if page_bytes == 0:
             return 1
         free, total = torch.cuda.mem_get_info(self.device)
@@ -157,12 +168,21 @@ class ModelRunner:
                 widest = max(widest, spec.shape[0])
         item = torch.empty((), dtype=self.dtype).element_size()
         activations = max_tokens * (3 * widest + 8 * s.hidden_size) * item + 2 * 512 * s.vocab_size * 4
-        budget = total * utilization - (total - free) - activations
+        # every recorded batch size keeps its own logits and a step's activations of that many rows
+        buckets = [b for b in self._bucket_sizes(graph_rows)] if graph_rows else []
+        recorded = sum(b * (s.vocab_size * 4 + (3 * widest + 8 * s.hidden_size) * item) + (64 << 20) for b in buckets)
+        budget = total * utilization - (total - free) - activations - recorded
         pages = int(budget // page_bytes)
         if pages <= 0:
             raise RuntimeError(f"no memory left for the cache: {free / 2**30:.1f} GiB free of {total / 2**30:.1f}, "
                                f"one page needs {page_bytes / 2**20:.1f} MiB")
         return pages
+
+    @staticmethod
+    def _bucket_sizes(largest: int) -> list[int]:
+        """Batch sizes that have a recorded step: powers of two and the sizes half way between, up to ``largest``."""
+        sizes = sorted({b for p in range(24) for b in (1 << p, 3 << p >> 1) if b >= 1})
+        return [b for b in sizes if b < largest] + [largest]
 
     # ------------------------------------------------------------------ the step
     def _fill_host_buffer(self, arrays: list[np.ndarray]) -> torch.Tensor:
@@ -207,16 +227,47 @@ class ModelRunner:
         """Reserves pages and lays the batch out as int32 arrays on the host.
         ``pad_to``: number of requests the arrays are made for (a graph's bucket; only for
         single-token entries): the padding rows store nothing and their results are dropped.
-        ``table_width``: fixed width of the block tables."""
+        ``table_width``: fixed width of the block tables.
+        Everything that can be wrong with the entries is found before anything is taken from the cache: a step
+        that is refused leaves no request admitted and no page reserved."""
         if not entries:
             raise ValueError("a step needs at least one entry")
+        cache = self.cache
         seen = set()
+        need = [0] * len(cache.groups)
+        new_requests = 0
         for e in entries:
             if e.request_id in seen:
                 raise ValueError(f"request {e.request_id!r} appears twice in one step")
             seen.add(e.request_id)
-            if len(e.tokens) == 0:
+            n = len(e.tokens)
+            if n == 0:
                 raise ValueError(f"request {e.request_id!r}: a step entry needs at least one token")
+            low, high = (e.tokens[0], e.tokens[0]) if n == 1 else (min(e.tokens), max(e.tokens))
+            if low < 0 or high >= self.vocab_size:
+                bad = low if low < 0 else high
+                raise ValueError(f"token id {bad} is outside the vocabulary of {self.vocab_size}")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its {n} tokens")
+            known = e.request_id in cache
+            new_requests += not known
+            new_len = (cache.num_tokens(e.request_id) if known else 0) + n
+            if new_len > self.max_position:
+                raise ValueError(f"request {e.request_id!r}: {new_len} tokens exceed the model's "
+                                 f"{self.max_position} positions")
+            for gi, g in enumerate(cache.groups):
+                if table_width is not None and -(-new_len // g.page_size) > table_width:
+                    raise ValueError(f"request {e.request_id!r}: {new_len} tokens need more than the {table_width} "
+                                     f"pages of {g.page_size} that max_model_len {self.max_model_len} allows")
+            for gi, k in enumerate(cache.pages_needed(e.request_id if known else None, new_len)):
+                need[gi] += k
+        for gi, k in enumerate(need):
+            if k > cache.num_free_pages(gi):
+                raise OutOfPages(f"group '{cache.groups[gi].name}': the step needs {k} more pages, "
+                                 f"{cache.num_free_pages(gi)} are free")
+        if new_requests > cache.num_free_slots():
+            raise OutOfPages(f"the step brings {new_requests} new requests, {cache.num_free_slots()} state slots are free")
         if all(len(e.tokens) == 1 for e in entries):
             return self._layout_single_tokens(entries, pad_to, table_width)
         return self._layout_general(entries, pad_to, table_width)
@@ -229,9 +280,6 @@ class ModelRunner:
                 cache.admit(e.request_id)
             start = cache.num_tokens(e.request_id)
             new_len = start + len(e.tokens)
-            if new_len > self.max_position:
-                raise ValueError(f"request {e.request_id!r}: {new_len} tokens exceed the model's "
-                                 f"{self.max_position} positions")
             cache.reserve(e.request_id, new_len)
             starts.append(start)
             new_lens.append(new_len)
@@ -242,34 +290,25 @@ class ModelRunner:
         T = int(q_lens.sum())
         cu = np.zeros(B + pad + 1, dtype=np.int32)
         np.cumsum(q_lens, out=cu[1:])
-        input_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries] + [np.zeros(pad, np.int64)])
-        if input_ids.min() < 0 or input_ids.max() >= self.vocab_size:
-            bad = int(input_ids[(input_ids < 0) | (input_ids >= self.vocab_size)][0])
-            raise ValueError(f"token id {bad} is outside the vocabulary of {self.vocab_size}")
-        input_ids = input_ids.astype(np.int32)
+        input_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries] + [np.zeros(pad, np.int32)])
         token_req = np.repeat(np.arange(B + pad, dtype=np.int32), q_lens)
         positions = (np.arange(T, dtype=np.int32) - np.repeat(cu[:-1], q_lens)
                      + np.repeat(np.array(starts + [0] * pad, dtype=np.int32), q_lens))
         context_lens = np.array(new_lens + [1] * pad, dtype=np.int32)
-        state_slots = np.array([cache.state_slot(e.request_id) for e in entries] + [0] * pad, dtype=np.int32)
-        rows = []
-        for i, e in enumerate(entries):
-            for w in e.want:
-                if not 0 <= w < len(e.tokens):
-                    raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
-                rows.append(int(cu[i]) + w)
+        # (padding rows work on the spare row of the state pools)
+        state_slots = np.array([cache.state_slot(e.request_id) for e in entries] + [self.num_state_slots] * pad,
+                               dtype=np.int32)
+        rows = [int(cu[i]) + w for i, e in enumerate(entries) for w in e.want]
 
         arrays = [input_ids, positions, token_req, cu, context_lens, state_slots]
         for gi, g in enumerate(cache.groups):
             tables = [cache.block_table(e.request_id, gi) for e in entries]
             width = table_width or max(1, max(len(t) for t in tables))
-            # padding rows point at page 0 (a place that exists) and store nothing (slot -1)
+            # padding rows read their one key on the spare page (zeros) and store nothing (slot -1)
             bt = np.full((B + pad, width), NO_PAGE, dtype=np.int32)
-            bt[B:, 0] = 0
+            bt[B:, 0] = self.num_pages
             slot_mapping = np.full(T, -1, dtype=np.int32)
             for i, t in enumerate(tables):
-                if len(t) > width:
-                    raise ValueError(f"request {entries[i].request_id!r} holds {len(t)} pages; the tables have {width}")
                 ta = np.asarray(t, dtype=np.int32)
                 bt[i, :len(t)] = ta
                 p = positions[cu[i]:cu[i + 1]]
@@ -294,46 +333,36 @@ class ModelRunner:
             if e.request_id not in cache:
                 cache.admit(e.request_id)
             start = cache.num_tokens(e.request_id)
-            if start + 1 > self.max_position:
-                raise ValueError(f"request {e.request_id!r}: {start + 1} tokens exceed the model's "
-                                 f"{self.max_position} positions")
-            token = e.tokens[0]
-            if not 0 <= token < self.vocab_size:
-                raise ValueError(f"token id {token} is outside the vocabulary of {self.vocab_size}")
             cache.reserve(e.request_id, start + 1)
             starts.append(start)
-            ids.append(token)
+            ids.append(e.tokens[0])
             slots.append(cache.state_slot(e.request_id))
-            for w in e.want:
-                if w != 0:
-                    raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its 1 tokens")
-                rows.append(i)
+            rows += [i] * len(e.want)
         n = B + pad
         new_lens = [s + 1 for s in starts]
         zeros = [0] * pad
         arrays = [np.array(ids + zeros, dtype=np.int32), np.array(starts + zeros, dtype=np.int32),
                   np.arange(n, dtype=np.int32), np.arange(n + 1, dtype=np.int32),
-                  np.array(new_lens + [1] * pad, dtype=np.int32), np.array(slots + zeros, dtype=np.int32)]
+                  np.array(new_lens + [1] * pad, dtype=np.int32),
+                  np.array(slots + [self.num_state_slots] * pad, dtype=np.int32)]
         for gi, g in enumerate(cache.groups):
             tables = [cache.block_table(e.request_id, gi) for e in entries]
             width = table_width or max(1, max(len(t) for t in tables))
-            # padding rows point at page 0 (a place that exists) and store nothing (slot -1)
+            # padding rows read their one key on the spare page (zeros) and store nothing (slot -1)
             flat, slot_mapping = [], [-1] * n
             ps = g.page_size
             for i, t in enumerate(tables):
-                if len(t) > width:
-                    raise ValueError(f"request {entries[i].request_id!r} holds {len(t)} pages; the tables have {width}")
                 flat += t
                 flat += [NO_PAGE] * (width - len(t))
                 page = t[starts[i] // ps]
                 if page == NO_PAGE:
                     raise RuntimeError(f"request {entries[i].request_id!r}: a new token falls on a page that was given back")
                 slot_mapping[i] = page * ps + starts[i] % ps
-            flat += ([0] + [NO_PAGE] * (width - 1)) * pad
+            flat += ([self.num_pages] + [NO_PAGE] * (width - 1)) * pad
             bt = np.array(flat, dtype=np.int32).reshape(n, width)
             arrays += [np.array(slot_mapping, dtype=np.int32), bt]
         meta = {"B": n, "T": n, "rows": rows, "starts": starts, "new_lens": new_lens, "q_lens": [1] * n,
-                "state_slots": slots + zeros, "max_q_len": 1, "max_context_len": max(new_lens)}
+                "state_slots": slots + [self.num_state_slots] * pad, "max_q_len": 1, "max_context_len": max(new_lens)}
         return arrays, meta
 
     def _context(self, dev: list[torch.Tensor], meta: dict, logit_rows: torch.Tensor | None, num_logit_rows: int,
@@ -363,8 +392,7 @@ class ModelRunner:
         """Runs the batch and returns float32 logits [wanted, vocab] in the order of the
         entries and of each entry's ``want`` (None if nothing is wanted). With ``keep=False`` the result may be
         memory that the next step overwrites (a caller that samples at once saves the copy)."""
-        if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)
-                and not self.state_pools):
+        if self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries):
             bucket = next(b for b in self.graph_buckets if b >= len(entries))
             if self._graphs.get(bucket, ...) is not None:
                 return self._graph_step(entries, bucket, keep)
@@ -394,8 +422,6 @@ class ModelRunner:
         buffer, and the bucket's graph (embedding to logits of every row) is replayed."""
         width = -(-self.max_model_len // self.page_size)
         arrays, meta = self._layout(entries, pad_to=bucket, table_width=width)
-        if meta["max_context_len"] > width * self.page_size:
-            raise ValueError(f"a request of {meta['max_context_len']} tokens exceeds max_model_len {self.max_model_len}")
         g = self._graphs.get(bucket)
         # a graph's kernels are laid out for the context lengths of the step that recorded it, g["planned"]; when the
         # longest context is half as long again, or less than half of it, a new graph is recorded (the old one is dropped)
@@ -403,7 +429,7 @@ class ModelRunner:
         longest = max(256, meta["max_context_len"])
         if g is None or not g["planned"] // 2 < longest <= g["planned"] + g["planned"] // 2:
             self.graphs_rerecorded += g is not None
-            g = self._capture(bucket, arrays, meta, width)
+            g = self._capture(bucket, arrays, meta, width, len(entries))
             self._graphs[bucket] = g if g["graph"] is not None else None
         if g["graph"] is not None:
             g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
@@ -423,7 +449,7 @@ class ModelRunner:
     def can_step_ahead(self, request_ids: list) -> bool:
         """Whether the next tokens of these requests can be run before the host knows them (``step_ahead``):
         a recorded graph for their number, laid out for their lengths, and a cache whose commits can be taken back."""
-        if not (self.use_graphs and request_ids and len(request_ids) <= self.max_graph_batch and not self.state_pools
+        if not (self.use_graphs and request_ids and len(request_ids) <= self.max_graph_batch
                 and not self.cache.share_prefixes and all(g.window is None for g in self.cache.groups)):
             return False
         g = self._graphs.get(next(b for b in self.graph_buckets if b >= len(request_ids)))
@@ -452,10 +478,18 @@ class ModelRunner:
         g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
         self._copy_issued()
         g["index"][:len(entries)].copy_(tokens[:len(entries)])     # the token ids are the first of the index arrays
+        # state of fixed size cannot be stepped back: what these requests' rows hold now is kept until the step's
+        # turn has come (a few rows per pool)
+        slots = meta["state_slots"][:len(entries)]
+        kept = None
+        if self.state_pools:
+            at = g["ctx"].state_slots[:len(entries)].long()
+            kept = [{name: t[at] for name, t in pool.items()} for pool in self.state_pools]
         g["graph"].replay()
         for e, n in zip(entries, meta["new_lens"]):
             self.cache.commit(e.request_id, n)
-        return {"requests": list(request_ids), "starts": meta["starts"], "logits": g["logits"]}
+        return {"requests": list(request_ids), "starts": meta["starts"], "logits": g["logits"], "slots": slots,
+                "kept_state": kept}
 
     def logits_ahead(self, ahead: dict, request_ids: list) -> torch.Tensor:
         """The logits of ``request_ids`` (some or all of the step's, in any order) from a step issued ahead."""
@@ -468,13 +502,24 @@ class ModelRunner:
         """Takes a step issued ahead back for these of its requests, as far as they still hold anything: their
         tokens count as not fed (the keys and values it stored are stored again, the same, when the step is run
         in its turn)."""
-        for r, start in zip(ahead["requests"], ahead["starts"]):
+        rows, slots = [], []
+        for i, (r, start) in enumerate(zip(ahead["requests"], ahead["starts"])):
             if r in request_ids and r in self.cache and self.cache.num_tokens(r) == start + 1:
                 self.cache.rewind(r, start)
+                rows.append(i)
+                slots.append(ahead["slots"][i])
+        if rows and ahead["kept_state"] is not None:
+            rows_t = torch.tensor(rows, device=self.device)
+            slots_t = torch.tensor(slots, device=self.device)
+            for pool, kept in zip(self.state_pools, ahead["kept_state"]):
+                for name, t in pool.items():
+                    t[slots_t] = kept[name][rows_t]
 
-    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int) -> dict:
+    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int, num_real: int) -> dict:
         """Runs the bucket's step once eagerly on its fixed buffers (so that every kernel library is loaded
-        and the allocator is warm), then records it, and checks the graph if a library call went into it."""
+        and the allocator is warm), then records it, and checks the graph if a library call went into it.
+        A model with per-request state is stepped several times here on the same tokens: the state that the
+        step found is put back before each run, so that all of them, and the caller's, start from it."""
         from ..native import ops
         sizes = [a.size for a in arrays]
         index = torch.zeros(sum(sizes), dtype=torch.int32, device=self.device)
@@ -496,6 +541,14 @@ class ModelRunner:
         # with other lengths stay right: the block tables and the splits' results are made for max_model_len)
         planned = max(256, meta["max_context_len"])
         backend.planned_context = planned
+        state_slots = ctx.state_slots.long()
+        found = [{name: t[state_slots] for name, t in pool.items()} for pool in self.state_pools]
+
+        def put_state_back():
+            for pool, rows in zip(self.state_pools, found):
+                for name, t in pool.items():
+                    t[state_slots] = rows[name]
+
         try:
             # warm-up; it writes the same cache slots as every replay will
             eager = self.model.logits(self.model.forward(ctx)).clone()
@@ -508,17 +561,21 @@ class ModelRunner:
                 print(f"[nanohybrid_vlm_amd] no graph for {bucket} requests ({str(err).splitlines()[0][:200]}); "
                       "steps of this size run eagerly", file=sys.stderr, flush=True)
                 return {"graph": None, "index": index, "logits": eager, "ctx": ctx, "planned": planned}
-            if with_library:
+            if with_library or self.state_pools:
                 for _ in range(3):
                     logits.fill_(float("nan"))
+                    put_state_back()
                     graph.replay()
                     torch.cuda.synchronize()
-                    if not self.graph_check(logits, eager):
+                    # (the rows of the requests: what the padding rows hold is nobody's result)
+                    if not self.graph_check(logits[:num_real], eager[:num_real]):
                         print(f"[nanohybrid_vlm_amd] the graph for {bucket} requests differs from the eager step when "
                               "replayed; steps of this size run eagerly", file=sys.stderr, flush=True)
                         return {"graph": None, "index": index, "logits": eager, "ctx": ctx, "planned": planned}
+                    put_state_back()
                     self.model.logits(self.model.forward(ctx))      # eager work between the replays
                     torch.cuda.synchronize()
+            put_state_back()                                  # the caller replays the graph for this very step
         finally:
             backend.own_kernels_only, backend.planned_context, backend.measure_linears = old
             if hasattr(backend, "end_measurements"):

@@ -196,7 +196,13 @@ class NativeBackend:
         split_len = 64
         while split_len * 2 <= want and split_len < 1024:
             split_len *= 2
-        n_splits = -(-batch.max_context_len // split_len)
+        # the splits cover the longest context this launch can meet: outside a graph the batch's own; inside one, half
+        # as much again as what was planned for (the recorder replaces a graph before its contexts outgrow that),
+        # not the bound of the block tables (max_model_len), whose splits would nearly all be empty blocks
+        covered = batch.max_context_len
+        if self.planned_context:
+            covered = min(covered, self.planned_context + self.planned_context // 2)
+        n_splits = -(-covered // split_len)
         part_o = torch.empty((T, Hq, n_splits, D), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, Hq, n_splits, 2), dtype=torch.float32, device=q.device)
         self._call("nhv_decode_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_o),

@@ -56,6 +56,12 @@ class CacheView:
 class Part:
     """Base of mixers, feed-forwards, norms, position encodings and blocks."""
 
+    # True: ``forward`` reads the step only through its device tensors and launches the same kernels whatever
+    # they hold, so a step can be recorded into a HIP graph and replayed. A part that loops over the step's
+    # host lists (``step.host``), or whose launches depend on values, says False; steps of a model with such a
+    # part always run eagerly.
+    recordable = True
+
     def param_specs(self) -> dict[str, ParamSpec]:
         return {}
 

@@ -47,6 +47,7 @@ class ModelSpec:
     max_position: int
     tie_embeddings: bool
     run_order: list[RunEntry] | None = None   # None: every layer once, in order
+    eos_token_id: int | None = None           # the token that ends a request, if the checkpoint names one
 
     def order(self) -> list[RunEntry]:
         if self.run_order is None:
@@ -108,6 +109,13 @@ class DecoderModel(Part):
         for p in self.positions.values():
             p.to(device)
         return self
+
+    def recordable(self) -> bool:
+        """Whether a step of this model can be recorded into a HIP graph and replayed with other index
+        tensors: every part works from the step's device tensors alone."""
+        def ok(part) -> bool:
+            return part.recordable and all(ok(c) for c in part.children().values())
+        return ok(self)
 
     # -- cache ------------------------------------------------------------
     def cache_needs(self) -> list[PagedKVNeed | StateNeed | None]:

@@ -24,10 +24,11 @@ from safetensors import safe_open
 class WeightsError(RuntimeError):
     """One error for everything that is wrong with a checkpoint."""
 
-    def __init__(self, folder, unexpected, missing, wrong_shape):
+    def __init__(self, folder, unexpected, missing, wrong_shape, differing=()):
         self.unexpected = list(unexpected)
         self.missing = list(missing)
         self.wrong_shape = list(wrong_shape)
+        self.differing = list(differing)
         lines = [f"the checkpoint in '{folder}' does not fit the model:"]
         if self.unexpected:
             lines.append(f"  unexpected tensors ({len(self.unexpected)}): " + ", ".join(self.unexpected))
@@ -35,6 +36,9 @@ class WeightsError(RuntimeError):
             lines.append(f"  missing tensors ({len(self.missing)}): " + ", ".join(self.missing))
         if self.wrong_shape:
             lines.append(f"  wrong shapes ({len(self.wrong_shape)}): " + "; ".join(self.wrong_shape))
+        if self.differing:
+            lines.append(f"  copies that differ from the tensor they repeat ({len(self.differing)}): "
+                         + "; ".join(self.differing))
         super().__init__("\n".join(lines))
 
 
@@ -54,7 +58,6 @@ def load_weights(model, arch, cfg, folder: str, dtype: torch.dtype, device) -> d
     and binds them to the model's parts. Returns the parameters by name."""
     specs = model.all_param_specs()
     sources = arch.checkpoint_names(cfg)
-    optional = set(arch.optional_names(cfg))
     for name, src in sources.items():
         if src.param not in specs:
             raise KeyError(f"architecture '{arch.name}' maps '{name}' to unknown parameter '{src.param}'")
@@ -68,8 +71,7 @@ def load_weights(model, arch, cfg, folder: str, dtype: torch.dtype, device) -> d
                 if any(key.startswith(p) for p in arch.ignored_prefixes):
                     continue
                 if key not in sources:
-                    if key not in optional:
-                        unexpected.append(key)
+                    unexpected.append(key)
                     continue
                 sl = f.get_slice(key)
                 shape = tuple(sl.get_shape())
@@ -79,15 +81,31 @@ def load_weights(model, arch, cfg, folder: str, dtype: torch.dtype, device) -> d
                 if shape != want:
                     wrong_shape.append(f"{key}: stored {list(shape)}, needed {list(want)}")
                 found[key] = (path, sl.get_dtype())
-    missing = [name for name in sources if name not in found and name not in optional]
-    if unexpected or missing or wrong_shape:
-        raise WeightsError(folder, sorted(unexpected), missing, wrong_shape)
+    missing = [name for name, src in sources.items() if name not in found and not src.copy]
+    # a stored copy (a tied head beside the embedding) must repeat its original: the reference copies it into the
+    # shared storage (nanovllm/models/qwen3.py:202-203), so a differing copy would silently replace the embedding
+    differing = []
+    originals = {(src.param, src.row_start, src.rows): name for name, src in sources.items() if not src.copy}
+    for name, src in sources.items():
+        if src.copy and name in found and not wrong_shape:
+            original = originals.get((src.param, src.row_start, src.rows))
+            if original is None or original not in found:
+                continue
+            with safe_open(found[name][0], framework="pt", device="cpu") as f:
+                a = f.get_tensor(name)
+            with safe_open(found[original][0], framework="pt", device="cpu") as f:
+                b = f.get_tensor(original)
+            if a.shape != b.shape or not torch.equal(a.to(torch.float32), b.to(torch.float32)):
+                differing.append(f"{name} is not equal to {original}")
+            del a, b
+    if unexpected or missing or wrong_shape or differing:
+        raise WeightsError(folder, sorted(unexpected), missing, wrong_shape, differing)
 
     # element type of every parameter
     params: dict[str, torch.Tensor] = {}
     by_param: dict[str, list[str]] = {}
     for name, src in sources.items():
-        if name in found:
+        if name in found and not src.copy:
             by_param.setdefault(src.param, []).append(name)
     for pname, spec in specs.items():
         stored = {found[n][1] for n in by_param.get(pname, [])}
@@ -102,7 +120,8 @@ def load_weights(model, arch, cfg, folder: str, dtype: torch.dtype, device) -> d
     # pass 2: copy, file by file
     by_file: dict[str, list[str]] = {}
     for name, (path, _) in found.items():
-        by_file.setdefault(path, []).append(name)
+        if not sources[name].copy:                       # (a copy was compared with its original above)
+            by_file.setdefault(path, []).append(name)
     for path, names in by_file.items():
         with safe_open(path, framework="pt", device="cpu") as f:
             for name in names:

@@ -38,6 +38,8 @@ def random_checkpoint_tensors(raw_config: dict, seed: int, store_dtype: str = "b
     specs = model.all_param_specs()
     out = {}
     for index, (name, src) in enumerate(arch.checkpoint_names(cfg).items()):
+        if src.copy:                                   # what a file may repeat is written once
+            continue
         spec = specs[src.param]
         shape = ((src.rows,) + tuple(spec.shape[1:])) if src.rows is not None else tuple(spec.shape)
         gen = torch.Generator(device="cpu")
@@ -73,7 +75,8 @@ def fill_random_on_device(model, seed: int, dtype: torch.dtype, device) -> dict[
     gen.manual_seed(int(seed))
     params = {}
     for name, spec in model.all_param_specs().items():
-        t = torch.empty(spec.shape, dtype=dtype, device=device)
+        # what a checkpoint would store in 32-bit (norm weights, routers) stays float32 here too
+        t = torch.empty(spec.shape, dtype=torch.float32 if spec.keeps_float32 else dtype, device=device)
         if spec.init == "norm":
             t.normal_(1.0, 0.1, generator=gen)
         else:
@@ -81,3 +84,17 @@ def fill_random_on_device(model, seed: int, dtype: torch.dtype, device) -> dict[
         params[name] = t
     model.bind_all(params)
     return params
+
+
+def build_random_model(raw_config: dict, seed: int, dtype: str | torch.dtype = "bfloat16", device="cuda:0"):
+    """(architecture, typed configuration, model with random weights bound) from config.json contents: what
+    ``ModelRunner`` and ``LLM`` take in place of a model folder. The weights are drawn on the device."""
+    from ..parts.model import DecoderModel
+
+    arch = resolve_architecture(raw_config)
+    cfg = arch.parse_config(raw_config)
+    model = DecoderModel(arch.build_spec(cfg))
+    if isinstance(dtype, str):
+        dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}[dtype]
+    fill_random_on_device(model, seed, dtype, device)
+    return arch, cfg, model

@@ -8,7 +8,8 @@ from safetensors.torch import load_file, save_file
 
 from conftest import TINY_A, TINY_B, TINY_C
 from nanohybrid_vlm_amd.config.engine_config import EngineConfig
-from nanohybrid_vlm_amd.config.model_config import ConfigError, Qwen3Config, read_config_json
+from nanohybrid_vlm_amd.architectures.qwen3 import Qwen3Config
+from nanohybrid_vlm_amd.config.model_config import ConfigError, read_config_json
 from nanohybrid_vlm_amd.config.registry import (Architecture, UnknownArchitecture, register_architecture,
                                                 resolve_architecture, unregister_architecture)
 from nanohybrid_vlm_amd.parts.model import DecoderModel

@@ -67,7 +67,10 @@ def test_padding_rows_store_nothing(runner):
     assert meta["B"] == 4 and meta["T"] == 4 and meta["rows"] == [0]
     assert a["bt"].shape == (4, 6)
     assert list(a["slot_mapping"][1:]) == [-1, -1, -1]              # nothing is stored for the padding
-    assert list(a["context_lens"][1:]) == [1, 1, 1] and (a["bt"][1:, 0] == 0).all()   # and they read a place that exists
+    # and they read one key on the spare page that no request is ever given, and work on the spare state row
+    assert list(a["context_lens"][1:]) == [1, 1, 1] and (a["bt"][1:, 0] == runner.num_pages).all()
+    assert runner.num_pages not in [p for r in runner.cache.requests.values() for t in r.tables for p in t]
+    assert list(a["state_slots"][1:]) == [runner.num_state_slots] * 3
     assert a["positions"][0] == 5 and a["slot_mapping"][0] == runner.cache.block_table("a")[1] * 4 + 1
 
 
@@ -83,7 +86,29 @@ def test_bad_entries_are_refused(runner):
     with pytest.raises(OutOfPages):
         runner._layout([StepEntry("c", [1] * 161, [])])
     runner.cache.check()
-    assert np.asarray(runner.cache.block_table("c")).size == 0     # all or nothing
+    assert "c" not in runner.cache                                 # all or nothing: not even admitted
+
+
+def test_a_refused_step_takes_nothing_from_the_cache(runner):
+    """Whatever is wrong with a later entry, the earlier ones are not admitted and hold no page."""
+    runner._layout([StepEntry("old", [1, 2, 3], [])])
+    runner.cache.commit("old", 3)
+    free, slots = runner.cache.num_free_pages(), runner.cache.num_free_slots()
+    good = StepEntry("new", [1] * 9, [8])
+    for bad, error in [(StepEntry("x", [runner.vocab_size + 3], []), ValueError),
+                       (StepEntry("x", [1, 2], [5]), ValueError),
+                       (StepEntry("x", [1] * (runner.max_position + 1), []), ValueError),
+                       (StepEntry("x", [1] * 4 * (free + 1), []), OutOfPages),
+                       (StepEntry("new", [4], []), ValueError)]:
+        with pytest.raises(error):
+            runner._layout([good, StepEntry("old", [7], [0]), bad])
+        runner.cache.check()
+        assert "new" not in runner.cache and "x" not in runner.cache
+        assert runner.cache.num_free_pages() == free and runner.cache.num_free_slots() == slots
+        assert runner.cache.num_tokens("old") == 3 and len(runner.cache.block_table("old")) == 1
+    with pytest.raises(ValueError, match="max_model_len"):
+        runner._layout([good, StepEntry("old", [7], [0])], table_width=2)
+    assert "new" not in runner.cache and runner.cache.num_free_pages() == free
 
 
 def test_graph_buckets_are_powers_of_two_and_the_sizes_half_way_up_to_the_limit(emulated_kernels, model_folders):
