@@ -16,10 +16,21 @@ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   return z ^ (z >> 31);
 }
 
+// Exp(1) noise from 24 random bits: -log(u) with u the middle of the bits' bucket, (bits + 0.5) / 2^24, so that
+// the smallest value, 3e-8, is the mean of what a true Exp(1) draw puts into the lowest bucket. (With u = (bits
+// + 1) / 2^24 the top pattern gave u = 1 and a noise of 0, held at 1e-10: once in 2^24 draws an index's chance was
+// multiplied by 10^10 where 3 * 10^7 is right, and with 150,000 indices a row that is one draw in a hundred.)
+// Both halves of the range are computed from numbers that float holds exactly: bits + 0.5 below 2^23, and
+// 1 - u = (2^24 - bits - 0.5) / 2^24 above, through log1p. The floor of 1e-10 is the reference's
+// (nanovllm/layers/sampler.py:52) and is never met.
+__device__ __forceinline__ float exp1_noise_of_bits(uint32_t bits) {
+  float e;
+  if (bits < (1u << 23)) e = -logf(((float)bits + 0.5f) * (1.0f / 16777216.0f));
+  else e = -log1pf(-((float)(16777216u - bits) - 0.5f) * (1.0f / 16777216.0f));
+  return fmaxf(e, 1e-10f);
+}
 __device__ __forceinline__ float exp1_noise(uint64_t key, int i) {
-  const uint32_t bits = (uint32_t)(mix64(key ^ (uint64_t)i) >> 40);      // 24 bits
-  const float u = (float)(bits + 1u) * (1.0f / 16777216.0f);             // (0, 1]
-  return fmaxf(-logf(u), 1e-10f);
+  return exp1_noise_of_bits((uint32_t)(mix64(key ^ (uint64_t)i) >> 40));   // 24 bits
 }
 
 struct Best {
@@ -112,6 +123,20 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   }
   best = block_best(best, bscratch);
   if (threadIdx.x == 0) tokens[blockIdx.x] = best.i;
+}
+
+__global__ void noise_of_bits_kernel(const uint32_t* __restrict__ bits, float* __restrict__ out, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = exp1_noise_of_bits(bits[i] & 0xFFFFFFu);
+}
+
+// the noise that each of n 24-bit patterns gives (for tests of the noise's distribution)
+extern "C" int nhv_noise_of_bits(const void* bits, void* out, int n, void* stream) {
+  NHV_REQUIRE(n > 0, "noise_of_bits: bad size n=%d", n);
+  hipLaunchKernelGGL(noise_of_bits_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                     (const uint32_t*)bits, (float*)out, n);
+  NHV_LAUNCH_CHECK("noise_of_bits");
+  return 0;
 }
 
 // how many floats (and as many ints) of scratch nhv_sample needs for n rows of V logits

@@ -107,6 +107,6 @@ class EmulatedBackend:
             noise = None
             if temp > 0:
                 key = int(keys[r]) & mask
-                noise = torch.tensor([-math.log(((mix(key ^ i) >> 40) + 1) / 16777216.0)
+                noise = torch.tensor([-math.log(((mix(key ^ i) >> 40) + 0.5) / 16777216.0)
                                       for i in range(logits.shape[1])], dtype=torch.float32)
             tokens[r] = sample_token(logits[r], temp, noise)

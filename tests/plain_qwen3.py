@@ -48,7 +48,7 @@ def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, 
 def rope_angles(positions: torch.Tensor, rotary_dim: int, base: float) -> torch.Tensor:
     """nanovllm/layers/rotary_embedding.py:83-85: inv_freq_j = base^(-2j/d),
     angle[p, j] = p * inv_freq_j, all in float32."""
-    inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+    inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32, device=positions.device) / rotary_dim))
     return positions.to(torch.float32)[:, None] * inv_freq[None, :]
 
 
@@ -77,8 +77,8 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
     T, Hq, D = q.shape
     Hkv = k.shape[1]
     group = Hq // Hkv
-    out = torch.empty(T, Hq, v.shape[-1], dtype=torch.float32)
-    pos = torch.arange(T)
+    out = torch.empty(T, Hq, v.shape[-1], dtype=torch.float32, device=q.device)
+    pos = torch.arange(T, device=q.device)
     allowed = pos[None, :] <= pos[:, None]
     if window is not None:
         allowed &= pos[None, :] > pos[:, None] - window
@@ -134,8 +134,9 @@ def attention_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: s
 def hidden_states(cfg: dict, w: dict, token_ids, first_position: int = 0) -> torch.Tensor:
     """nanovllm/models/qwen3.py:152-159 and :178-182, written as the usual
     pre-norm block: r += attn(norm(r)); r += mlp(norm(r)); final norm."""
-    ids = torch.as_tensor(token_ids, dtype=torch.long)
-    positions = torch.arange(first_position, first_position + ids.numel())
+    device = w["model.embed_tokens.weight"].device          # (the tensors may be moved to another device as they are)
+    ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
+    positions = torch.arange(first_position, first_position + ids.numel(), device=device)
     eps = cfg["rms_norm_eps"]
     assert cfg.get("hidden_act", "silu") == "silu"               # qwen3.py:110
     r = w["model.embed_tokens.weight"][ids]                      # embed_head.py:38
@@ -175,8 +176,8 @@ def greedy_generate(cfg: dict, w: dict, prompt, n_new: int, eos: int | None = No
 def sample_noise(seed: int, request: int, step: int, n: int) -> torch.Tensor:
     """The engine's own counter-based noise (no counterpart in the reference,
     which draws from torch's global generator, nanovllm/layers/sampler.py:50-54):
-    uniform u in (0, 1] from a 64-bit mix of (seed, request, step, index), then
-    Exp(1) noise -log(u). Written here independently, in Python integers."""
+    24 bits from a 64-bit mix of (seed, request, step, index), then Exp(1) noise
+    ``noise_of_bits``. Written here independently, in Python integers."""
     mask = (1 << 64) - 1
 
     def mix(z):
@@ -188,10 +189,13 @@ def sample_noise(seed: int, request: int, step: int, n: int) -> torch.Tensor:
     key = mix(mix(mix(seed & mask) ^ (request & mask)) ^ (step & mask))
     out = torch.empty(n, dtype=torch.float32)
     for i in range(n):
-        bits = mix(key ^ i) >> 40                       # 24 random bits
-        u = (bits + 1) * (1.0 / 16777216.0)             # (0, 1]
-        out[i] = -math.log(u)
+        out[i] = noise_of_bits(mix(key ^ i) >> 40)      # 24 random bits
     return out
+
+
+def noise_of_bits(bits: int) -> float:
+    """-log(u) with u = (bits + 0.5) / 2^24, the middle of the bucket of the 24 bits, in double precision."""
+    return -math.log((bits + 0.5) / 16777216.0)
 
 
 def sample_token(logits_row: torch.Tensor, temperature: float, noise: torch.Tensor | None) -> int:

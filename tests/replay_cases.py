@@ -104,20 +104,8 @@ def peak_tokens(steps: list[dict], page: int = 64) -> int:
 
 
 def run_in_process(runner, steps: list[dict]) -> dict[str, torch.Tensor]:
-    """Drives ``runner.step`` with a trace; returns per request the logits of all its tokens, in order."""
-    from nanohybrid_vlm_amd.engine.runner import StepEntry
+    """A trace through the replay program's own function, in this process: per request the logits of all its
+    tokens, in order."""
+    from nanohybrid_vlm_amd.engine.replay import replay
 
-    out: dict[str, list[torch.Tensor]] = {}
-    for st in steps:
-        entries = [StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]]
-        logits = runner.step(entries)
-        row = 0
-        for e in st["entries"]:
-            n = len(e["want"])
-            if n:
-                out.setdefault(e["id"], []).append(logits[row:row + n].float().cpu())
-                row += n
-        for rid in st["end"]:
-            runner.finish(rid)
-        runner.cache.check()
-    return {rid: torch.cat(parts) for rid, parts in out.items()}
+    return replay(runner, steps)

@@ -120,7 +120,19 @@ def test_tied_head_and_bias(tmp_path):
     # a tied checkpoint that repeats the embedding as lm_head.weight is accepted too
     stored["lm_head.weight"] = stored["model.embed_tokens.weight"].clone()
     save_file(stored, os.path.join(folder, "model.safetensors"))
-    _load(folder)
+    model, params = _load(folder)
+    assert model.head_weight is model.embed_weight and torch.equal(params["embed.weight"], stored["model.embed_tokens.weight"].float())
+    # but a copy that differs from the embedding is an error, not a silent choice between the two
+    # (the reference copies it over the shared storage, nanovllm/models/qwen3.py:202-203)
+    stored["lm_head.weight"][3, 5] += 0.25
+    save_file(stored, os.path.join(folder, "model.safetensors"))
+    with pytest.raises(WeightsError, match="lm_head.weight is not equal to model.embed_tokens.weight") as info:
+        _load(folder)
+    assert info.value.differing and not info.value.missing and not info.value.unexpected
+    stored["lm_head.weight"] = torch.zeros(7, 64, dtype=torch.bfloat16)
+    save_file(stored, os.path.join(folder, "model.safetensors"))
+    with pytest.raises(WeightsError, match="wrong shapes"):
+        _load(folder)
     folder = write_random_model(str(tmp_path / "c"), TINY_C, seed=2)
     model, params = _load(folder)
     assert "layers.0.mixer.qkv.bias" in params and "layers.0.mixer.q_norm.weight" not in params
@@ -163,6 +175,56 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     msg = str(e)
     for piece in ("missing", "unexpected", "wrong shapes", "k_proj", "extra_proj", "needed [96, 160]"):
         assert piece in msg
+
+
+def test_ignored_prefixes_are_skipped(tmp_path):
+    """Tensors under a prefix that the architecture declares ignored (a vision tower beside the decoder, say) are
+    neither loaded nor reported (nanovllm/utils/loader.py:27-31,85-93)."""
+    import dataclasses
+    from nanohybrid_vlm_amd.architectures.qwen3 import QWEN3
+    from nanohybrid_vlm_amd.parts.model import DecoderModel
+    from nanohybrid_vlm_amd.weights.loader import load_weights
+    folder = write_random_model(str(tmp_path / "m"), TINY_A, seed=0)
+    path = os.path.join(folder, "model.safetensors")
+    stored = load_file(path)
+    stored["visual.blocks.0.weight"] = torch.zeros(3, 3)
+    stored["mtp.head.weight"] = torch.zeros(2)
+    save_file(stored, path)
+    with pytest.raises(WeightsError) as info:
+        _load(folder)
+    assert info.value.unexpected == ["mtp.head.weight", "visual.blocks.0.weight"]
+    arch = dataclasses.replace(QWEN3, ignored_prefixes=("visual.", "mtp."))
+    cfg = arch.parse_config(TINY_A)
+    model = DecoderModel(arch.build_spec(cfg))
+    params = load_weights(model, arch, cfg, folder, torch.float32, "cpu")
+    assert "embed.weight" in params and not any("visual" in n or "mtp" in n for n in params)
+
+
+def test_a_nested_text_config_is_read(tmp_path):
+    """A multimodal checkpoint nests the decoder's keys under text_config (nanovllm/config.py:318-322)."""
+    nested = {"architectures": ["Qwen3ForCausalLM"], "vision_config": {"hidden_size": 11},
+              "text_config": {k: v for k, v in TINY_B.items() if k != "architectures"}}
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(nested, f)
+    raw = read_config_json(str(tmp_path))
+    cfg = Qwen3Config.from_dict(raw)
+    assert cfg.hidden_size == 96 and cfg.architectures == ("Qwen3ForCausalLM",) and cfg.model_type == "qwen3"
+    # keys at the top level win: a plain config.json that happens to carry a text_config is read as it is
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(dict(TINY_A, text_config={"hidden_size": 1}), f)
+    assert Qwen3Config.from_dict(read_config_json(str(tmp_path))).hidden_size == 64
+
+
+def test_random_weights_on_the_device_keep_float32_tensors():
+    """Weights drawn in place of a checkpoint: what a checkpoint would keep in 32-bit (norm weights) is float32,
+    the matrices have the run's element type."""
+    from nanohybrid_vlm_amd.weights.random_init import build_random_model
+    arch, cfg, model = build_random_model(TINY_B, seed=5, dtype="bfloat16", device="cpu")
+    specs = model.all_param_specs()
+    for name, t in model.parameters.items():
+        assert t.dtype == (torch.float32 if specs[name].keeps_float32 else torch.bfloat16), name
+    assert abs(model.parameters["final_norm.weight"].mean().item() - 1.0) < 0.1
+    assert model.parameters["embed.weight"].float().std().item() == pytest.approx(0.02, rel=0.1)
 
 
 def test_missing_files(tmp_path):

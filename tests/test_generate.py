@@ -218,3 +218,102 @@ def test_steps_issued_ahead_change_no_token(model_folders):
             if pages == 14:
                 assert llm.scheduler.num_preemptions > 0, "the small cache was meant to force a request out"
         assert ahead_steps[False] == 0 and ahead_steps[True] >= 10
+
+
+def _near_best(cfg, w, prompt, tokens, slack=2e-2):
+    """Every generated token is one the plain implementation rates within ``slack`` of its best, given the tokens
+    before it (bfloat16 may choose the other of two nearly equal logits; from there on the run is its own)."""
+    ids = list(prompt)
+    for t in tokens:
+        row = plain.logits(cfg, w, ids)[-1]
+        assert row[t] >= row.max() - slack, "a token far from the best was chosen"
+        ids.append(t)
+
+
+@pytest.mark.gpu
+def test_steps_issued_ahead_and_recomputation_in_bfloat16(model_folders):
+    """In bfloat16 a recorded step may hold the library's matrix products: the tokens with steps issued ahead are
+    bit for bit those without (the same recorded steps run either way), with ample pages and with so few that
+    requests are pushed out and computed again; and every token is one the plain implementation rates best or
+    nearly so."""
+    folder = model_folders["B"]
+    cfg, w = plain.read_model_folder(folder)
+    V = cfg["vocab_size"]
+    prompts = [random_tokens(V, n, 190 + n) for n in (3, 9, 20, 31, 40, 2)]
+    params = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True) for n in (24, 30, 20, 1, 2, 17)]
+    for pages in (64, 14):
+        runs = {}
+        for run_ahead in (False, True):
+            llm = LLM(folder, dtype="bfloat16", kvcache_block_size=8, num_kvcache_blocks=pages, max_num_batched_tokens=16,
+                      run_ahead=run_ahead)
+            done = {}
+            for p, sp in zip(prompts[:3], params[:3]):
+                llm.add_request(p, sp)
+            for _ in range(9):
+                done.update(llm.step()[0])
+            for p, sp in zip(prompts[3:], params[3:]):
+                llm.add_request(p, sp)
+            while not llm.is_finished():
+                done.update(llm.step()[0])
+            runs[run_ahead] = [done[i] for i in range(len(prompts))]
+            llm.runner.cache.check()
+            assert llm.get_memory_stats()["groups"][0]["free_pages"] == pages
+            assert (llm.num_steps_ahead >= 10) == run_ahead
+            if pages == 14:
+                assert llm.scheduler.num_preemptions > 0, "the small cache was meant to force a request out"
+        assert runs[True] == runs[False], f"{pages} pages: steps issued ahead changed a token"
+        for p, sp, tokens in zip(prompts, params, runs[True]):
+            assert len(tokens) == sp.max_tokens
+            _near_best(cfg, w, p, tokens)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cache_sized_from_free_memory(model_folders, dtype):
+    """``num_kvcache_blocks=-1`` (the default): the pages are what is left of ``gpu_memory_utilization`` of the
+    device's memory after the weights, the state pools, a step's activations and the recorded steps
+    (nanovllm/engine/model_runner.py:654-699). The device then holds no more than that share, and generation
+    is right."""
+    folder = model_folders["B"]
+    cfg, w = plain.read_model_folder(folder)
+    free_before, total = torch.cuda.mem_get_info()
+    share = min(0.9, (total - free_before) / total + 0.04)           # what is in use already and 4 % of the device more
+    llm = LLM(folder, dtype=dtype, kvcache_block_size=256, gpu_memory_utilization=share, max_num_batched_tokens=512,
+              max_model_len=512)
+    stats = llm.get_memory_stats()
+    pages = stats["groups"][0]["pages"]
+    assert llm.config.num_kvcache_blocks == pages > 0
+    item = 4 if dtype == "float32" else 2
+    page_bytes = 2 * 256 * cfg["num_key_value_heads"] * cfg["head_dim"] * item * cfg["num_hidden_layers"]
+    assert stats["kv_cache_bytes"] == pages * page_bytes
+    # most of the 4 % went to pages, and the device's share is kept
+    assert 0.5 * 0.04 * total <= stats["kv_cache_bytes"] <= 0.04 * total
+    assert total - stats["device_free_bytes"] <= share * total
+    prompts = [random_tokens(cfg["vocab_size"], n, 300 + n) for n in (300, 5, 260)]
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True), use_tqdm=False)
+    for p, o in zip(prompts, outs):
+        if dtype == "float32":
+            assert o["token_ids"] == plain.greedy_generate(cfg, w, p, 6)
+        else:
+            _near_best(cfg, w, p, o["token_ids"])
+    assert total - torch.cuda.mem_get_info()[0] <= share * total + (256 << 20), "generation stayed within the share (and the allocator's slack)"
+    with pytest.raises(RuntimeError, match="no memory left for the cache"):
+        LLM(folder, dtype=dtype, kvcache_block_size=256, gpu_memory_utilization=max(0.001, (total - free_before) / total * 0.5))
+
+
+def test_a_configuration_with_random_weights_in_place_of_a_folder(emulated_kernels):
+    """``LLM(config.json contents, random_weights=seed)``: a model of that configuration with weights drawn in
+    place; the same seed gives the same model."""
+    from conftest import TINY_B
+    sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    options = dict(device="cpu", dtype="float32", kvcache_block_size=4, num_kvcache_blocks=32, max_model_len=64)
+    runs = [LLM(dict(TINY_B), random_weights=seed, **options).generate([[5, 17, 3], [9, 200, 31, 7] * 3], sp, use_tqdm=False)
+            for seed in (3, 3, 4)]
+    assert runs[0] == runs[1] and runs[0] != runs[2]
+    assert LLM(dict(TINY_B), random_weights=3, **options).config.eos == TINY_B["eos_token_id"]
+    with pytest.raises(TypeError, match="needs random_weights"):
+        LLM(dict(TINY_B), **options)
+    with pytest.raises(TypeError, match="goes with a configuration"):
+        LLM("some folder", random_weights=1, **options)
+    with pytest.raises(ValueError, match="dtype"):
+        LLM(dict(TINY_B), random_weights=1, device="cpu", dtype="float16")

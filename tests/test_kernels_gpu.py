@@ -418,7 +418,7 @@ def test_sampling(ops, V):
         for r in range(2, n):
             key = int(keys[r]) & mask
             # the noise of plain_qwen3.sample_noise for an already mixed key
-            noise = torch.tensor([-math.log(((_mix(key ^ i) >> 40) + 1) / 16777216.0) for i in range(V)])
+            noise = torch.tensor([plain.noise_of_bits(_mix(key ^ i) >> 40) for i in range(V)])
             assert tokens[r] == plain.sample_token(logits[r].cpu(), float(temps[r]), noise)
 
 
@@ -428,6 +428,27 @@ def _mix(z):
     z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
     z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
     return z ^ (z >> 31)
+
+
+def test_noise_of_every_bit_pattern(ops):
+    """All 2^24 patterns through the kernel's own noise function: the values are those of the plain formula, none is
+    0 or infinite, and the share of patterns below x is the Exp(1) distribution's 1 - exp(-x) to within one
+    pattern, from the smallest values (3e-8) up. A noise of 1e-10 once in 2^24 draws would fail both."""
+    import ctypes
+    import numpy as np
+    n = 1 << 24
+    bits = torch.arange(n, dtype=torch.int32, device="cuda")
+    out = torch.empty(n, dtype=torch.float32, device="cuda")
+    lib = ops.backend().lib
+    assert lib.nhv_noise_of_bits(ctypes.c_void_p(bits.data_ptr()), ctypes.c_void_p(out.data_ptr()), n,
+                                 ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    got = out.cpu().numpy().astype(np.float64)
+    want = -np.log((np.arange(n, dtype=np.float64) + 0.5) / n)
+    assert np.isfinite(got).all() and got.min() > 2.9e-8
+    assert np.abs(got / want - 1).max() < 1e-6
+    ordered = np.sort(got)
+    share = np.arange(1, n + 1) / n                       # share of patterns at or below each value
+    assert np.abs(share - (1 - np.exp(-ordered))).max() <= 1.01 / n
 
 
 def test_sampling_follows_the_distribution(ops):

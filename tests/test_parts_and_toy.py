@@ -1,250 +1,174 @@
-"""The parts are general: a toy architecture, defined here and nowhere in the package,
-with a mixer that keeps state of its own per request, a feed-forward that routes every
-token to one of several experts, a position encoding of its own (other angles, on a
-part of the head only), a layer with a window (pages of its own, given back as the
-window passes), a layer that runs twice and an entry that reads another entry's cache,
-is registered, built, loaded and stepped through the unchanged engine and compared
+"""The parts are general: a toy architecture, defined in the tests and nowhere in the package
+(``toy_architecture.py``), is registered, built, loaded and stepped through the unchanged
+engine (the step function, the scheduler, the entry point, the command line) and compared
 with a plain whole-sequence computation.
 Also: each built-in part alone against its plain function."""
+import json
+import os
+import subprocess
+import sys
+
 import pytest
 import torch
 
 import plain_qwen3 as plain
 import replay_cases as rc
+import toy_architecture as toy
 from helpers import max_abs_diff
 from nanohybrid_vlm_amd.cache.manager import NO_PAGE
-from nanohybrid_vlm_amd.config.registry import (Architecture, WeightSource, register_architecture,
-                                                unregister_architecture)
-from nanohybrid_vlm_amd.parts import FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, ParamSpec, Part, StateNeed
-from nanohybrid_vlm_amd.parts.model import DecoderModel, LayerSpec, ModelSpec, RunEntry
+from nanohybrid_vlm_amd.parts.model import DecoderModel, RunEntry
 from nanohybrid_vlm_amd.weights.random_init import write_random_model
+from toy_architecture import VOCAB, WINDOW, toy_plain_logits, toy_spec
 
-H, HEADS, KV, D, INTER, VOCAB, WINDOW, DECAY = 48, 3, 1, 16, 64, 97, 5, 0.75
-EXPERTS, EXPERT_INTER, TOY_ROT, TOY_STEP = 3, 40, 8, 0.05
-
-
-class DecayingSum(Part):
-    """Toy mixer with state: s_t = decay * s_(t-1) + x_t per request, output s_t W^T.
-    The state of a request lives in its state slot between steps."""
-
-    def __init__(self, hidden_size: int, decay: float, position=None):
-        self.hidden_size, self.decay = hidden_size, decay
-
-    def param_specs(self):
-        return {"out.weight": ParamSpec((self.hidden_size, self.hidden_size))}
-
-    def bind(self, params):
-        self.weight = params["out.weight"]
-
-    def cache_need(self):
-        return StateNeed({"sum": ((self.hidden_size,), torch.float32)})
-
-    def forward(self, x, step, cache):
-        pool = cache.state["sum"]
-        out = torch.empty_like(x)
-        t = 0
-        for start, n, slot in zip(step.host["starts"], step.host["q_lens"], step.host["state_slots"]):
-            s = torch.zeros_like(pool[slot]) if start == 0 else pool[slot].clone()   # a new request starts from zero
-            for i in range(n):
-                s = self.decay * s + x[t + i].float()
-                out[t + i] = (s @ self.weight.float().T).to(x.dtype)
-            pool[slot] = s
-            t += n
-        return out
-
-
-class RoutedFeedForward(Part):
-    """Toy feed-forward with routing: router logits and their softmax in float32; every token goes through
-    the expert it rates highest (the experts are the package's own gated feed-forwards, built through the
-    registry) and the result is weighted with that expert's probability."""
-
-    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int):
-        self.hidden_size = hidden_size
-        self.experts = [FEED_FORWARDS.build({"kind": "swiglu", "hidden_size": hidden_size,
-                                             "intermediate_size": intermediate_size}) for _ in range(num_experts)]
-
-    def param_specs(self):
-        return {"router.weight": ParamSpec((len(self.experts), self.hidden_size), keeps_float32=True)}
-
-    def children(self):
-        return {f"experts.{i}": e for i, e in enumerate(self.experts)}
-
-    def bind(self, params):
-        self.router = params["router.weight"]
-
-    def forward(self, x, step):
-        prob = torch.softmax(x.float() @ self.router.float().T, dim=-1)
-        best = prob.argmax(dim=-1)
-        out = torch.zeros_like(x)
-        for e, expert in enumerate(self.experts):
-            rows = (best == e).nonzero().flatten()
-            if rows.numel():
-                y = expert.forward(x[rows].contiguous(), step)
-                out[rows] = (y.float() * prob[rows, e:e + 1]).to(x.dtype)
-        return out
-
-
-class LinearAngles(Part):
-    """Toy position encoding: the angle of pair j at position p is p * (j + 1) * step, and only the first
-    ``rotary_dim`` entries of a head are turned."""
-
-    def __init__(self, rotary_dim: int, step: float, max_position: int, device=None):
-        ang = torch.arange(max_position, dtype=torch.float32)[:, None] * (torch.arange(rotary_dim // 2) + 1.0) * step
-        self.table = torch.cat((ang.cos(), ang.sin()), dim=-1).contiguous()
-
-    def rotation_table(self):
-        return self.table
-
-    def to(self, device):
-        self.table = self.table.to(device)
-        return self
-
-
-def toy_spec(cfg: dict) -> ModelSpec:
-    norm = {"kind": "rmsnorm", "size": H, "eps": 1e-5}
-    ff = {"kind": "swiglu", "hidden_size": H, "intermediate_size": INTER}
-
-    def attention(window):
-        return {"kind": "gqa_attention", "hidden_size": H, "num_heads": HEADS, "num_kv_heads": KV, "head_dim": D,
-                "scale": D ** -0.5, "qk_norm_eps": 1e-5, "qkv_bias": False, "window": window}
-    routed = {"kind": "toy_routed", "hidden_size": H, "intermediate_size": EXPERT_INTER, "num_experts": EXPERTS}
-    layers = [
-        LayerSpec(mixer=attention(None), feed_forward=ff, norm=norm),
-        LayerSpec(mixer={"kind": "toy_decaying_sum", "hidden_size": H, "decay": DECAY}, feed_forward=routed, norm=norm),
-        LayerSpec(mixer=attention(WINDOW), feed_forward=ff, norm=norm, position="linear"),
-    ]
-    # layer 0 runs twice (two caches); the last entry runs layer 2 again on the keys and values of entry 2
-    order = [RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(2, cache=2)]
-    return ModelSpec(vocab_size=VOCAB, hidden_size=H, layers=layers, final_norm=norm,
-                     positions={"default": {"kind": "rope", "rotary_dim": D, "base": 1000.0},
-                                "linear": {"kind": "toy_linear_angles", "rotary_dim": TOY_ROT, "step": TOY_STEP}},
-                     max_position=256, tie_embeddings=True, run_order=order)
-
-
-def toy_names(cfg):
-    return {name: WeightSource(name) for name in DecoderModel(toy_spec(cfg)).all_param_specs()}
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 @pytest.fixture()
 def toy_architecture():
-    _register_toy_parts()
-    register_architecture(Architecture("ToyForCausalLM", ("toy",), dict, toy_spec, toy_names))
+    toy.register()
     yield
-    unregister_architecture("ToyForCausalLM")
-    _unregister_toy_parts()
+    toy.unregister()
 
 
-def _register_toy_parts():
-    MIXERS.register("toy_decaying_sum")(DecayingSum)
-    FEED_FORWARDS.register("toy_routed")(RoutedFeedForward)
-    POSITION_ENCODINGS.register("toy_linear_angles")(LinearAngles)
+def _toy_folder(tmp_path, device_state=False, **keys):
+    cfg = {"architectures": ["ToyForCausalLM"], "model_type": "toy", "device_state": device_state, **keys}
+    return write_random_model(str(tmp_path / f"toy{int(device_state)}"), cfg, seed=4)
 
 
-def _unregister_toy_parts():
-    MIXERS.unregister("toy_decaying_sum")
-    FEED_FORWARDS.unregister("toy_routed")
-    POSITION_ENCODINGS.unregister("toy_linear_angles")
-
-
-def toy_turn(x, pos):
-    """The toy position encoding on [T, heads, D]: pairs (j, j + TOY_ROT / 2) of the first TOY_ROT entries."""
-    ang = pos.float()[:, None] * (torch.arange(TOY_ROT // 2) + 1.0) * TOY_STEP
-    cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
-    x1, x2 = x[..., :TOY_ROT // 2], x[..., TOY_ROT // 2:TOY_ROT]
-    return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., TOY_ROT:]), dim=-1)
-
-
-def toy_plain_logits(w, toks):
-    """Whole sequence, no cache, from the plain functions."""
-    T = len(toks)
-    pos = torch.arange(T)
-    r = w["embed.weight"][toks]
-    kept = {}
-
-    def attention(x, p, window, entry, lender=None):
-        turn = toy_turn if window else (lambda t, at: plain.apply_rope(t, at, 1000.0))   # the windowed layer has the toy angles
-        qkv = x @ w[p + "mixer.qkv.weight"].T
-        q = plain.rms_norm(qkv[:, :HEADS * D].view(T, HEADS, D), w[p + "mixer.q_norm.weight"], 1e-5)
-        if lender is None:
-            k = plain.rms_norm(qkv[:, HEADS * D:(HEADS + KV) * D].view(T, KV, D), w[p + "mixer.k_norm.weight"], 1e-5)
-            v = qkv[:, (HEADS + KV) * D:].view(T, KV, D)
-            kept[entry] = (turn(k, pos), v)
-        k, v = kept[entry if lender is None else lender]
-        o = plain.causal_attention(turn(q, pos), k, v, D ** -0.5, window)
-        return o.reshape(T, HEADS * D) @ w[p + "mixer.o.weight"].T
-
-    def routed(x, p):
-        prob = torch.softmax(x @ w[p + "feed_forward.router.weight"].T, dim=-1)
-        rows = []
-        for t in range(T):
-            e = int(prob[t].argmax())
-            gu = w[p + f"feed_forward.experts.{e}.gate_up.weight"]
-            y = plain.swiglu(x[t:t + 1], gu[:EXPERT_INTER], gu[EXPERT_INTER:], w[p + f"feed_forward.experts.{e}.down.weight"])
-            rows.append(y[0] * prob[t, e])
-        return torch.stack(rows)
-
-    def decaying_sum(x, p):
-        s, rows = torch.zeros(H), []
-        for t in range(T):
-            s = DECAY * s + x[t]
-            rows.append(s @ w[p + "mixer.out.weight"].T)
-        return torch.stack(rows)
-
-    for entry, (layer, lender) in enumerate([(0, None), (1, None), (2, None), (0, None), (2, 2)]):
-        p = f"layers.{layer}."
-        x = plain.rms_norm(r, w[p + "mixer_norm.weight"], 1e-5)
-        if layer == 1:
-            r = r + decaying_sum(x, p)
-        else:
-            r = r + attention(x, p, WINDOW if layer == 2 else None, entry, lender)
-        x = plain.rms_norm(r, w[p + "feed_forward_norm.weight"], 1e-5)
-        if layer == 1:
-            r = r + routed(x, p)
-            continue
-        gu = w[p + "feed_forward.gate_up.weight"]
-        r = r + plain.swiglu(x, gu[:INTER], gu[INTER:], w[p + "feed_forward.down.weight"])
-    return plain.rms_norm(r, w["final_norm.weight"], 1e-5) @ w["embed.weight"].T
-
-
-def _toy_check(device, dtype, tol, tmp_path):
-    from nanohybrid_vlm_amd.engine.runner import ModelRunner
-    cfg = {"architectures": ["ToyForCausalLM"], "model_type": "toy"}
-    folder = write_random_model(str(tmp_path / "toy"), cfg, seed=4)
+def _toy_check(device, dtype, tol, tmp_path, device_state=False, graphs=False):
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner, StepEntry
+    folder = _toy_folder(tmp_path, device_state)
     _, w = plain.read_model_folder(folder)
     requests = {f"r{i}": rc.random_tokens(VOCAB, n, 30 + i) for i, n in enumerate([9, 40, 23, 17, 31])}
     want = {rid: toy_plain_logits(w, toks) for rid, toks in requests.items()}
     for mode, steps in [("whole", rc.whole(requests)), ("portions", rc.portions(requests)),
-                        ("mixed", rc.mixed(requests, max_live=3))]:
+                        ("tail", rc.tail_decoded(requests, tail=12)), ("mixed", rc.mixed(requests, max_live=3))]:
         pages = rc.peak_tokens(steps, 4) // 4
-        runner = ModelRunner(folder, dtype=dtype, device=device, page_size=4, num_pages=pages, num_state_slots=3)
+        runner = ModelRunner(folder, dtype=dtype, device=device, page_size=4, num_pages=pages, num_state_slots=3,
+                             use_graphs=graphs, max_model_len=64)
         assert len(runner.cache.groups) == 2 and runner.cache.groups[1].window == WINDOW
         assert len(runner.kv_tensors) == 3 and len(runner.state_pools) == 1       # entries 0, 2, 3 store keys; entry 1 state
+        # a part that walks over the step's requests on the host keeps the whole model out of graphs
+        assert runner.use_graphs == (graphs and device_state)
         got = rc.run_in_process(runner, steps)
         for rid in requests:
             d = max_abs_diff(got[rid], want[rid])
             assert d <= tol, f"toy {mode}: request {rid}: {d:.3e}"
         assert all(runner.cache.num_free_pages(g) == pages for g in range(2))
+        if runner.use_graphs and mode in ("tail", "mixed"):
+            stats = runner.get_memory_stats()
+            assert stats["graphs_recorded"] and not stats["graphs_refused"], stats
     # the windowed group gives pages back while a request is still alive
     runner = ModelRunner(folder, dtype=dtype, device=device, page_size=4, num_pages=16, num_state_slots=3)
-    from nanohybrid_vlm_amd.engine.runner import StepEntry
     runner.step([StepEntry("x", requests["r1"][:30], [29])])
     assert runner.cache.block_table("x", 0).count(NO_PAGE) == 0
     assert runner.cache.block_table("x", 1).count(NO_PAGE) == (30 - WINDOW + 1) // 4
 
 
-def test_toy_architecture_on_emulated_kernels(toy_architecture, emulated_kernels, tmp_path):
-    _toy_check("cpu", "float32", 2e-5, tmp_path)
+@pytest.mark.parametrize("device_state", [False, True], ids=["state on the host", "state on the device"])
+def test_toy_architecture_on_emulated_kernels(toy_architecture, emulated_kernels, tmp_path, device_state):
+    _toy_check("cpu", "float32", 2e-5, tmp_path, device_state)
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("device_state,graphs", [(False, False), (False, True), (True, True)],
+                         ids=["state on the host", "state on the host, graphs asked for", "state on the device, graphs"])
 @pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
-def test_toy_architecture_on_gpu(toy_architecture, dtype, tol, tmp_path):
-    _toy_check("cuda:0", dtype, tol, tmp_path)
+def test_toy_architecture_on_gpu(toy_architecture, dtype, tol, tmp_path, device_state, graphs):
+    _toy_check("cuda:0", dtype, tol, tmp_path, device_state, graphs)
+
+
+def _toy_greedy(w, prompt, n, eos=None):
+    ids, out = list(prompt), []
+    for _ in range(n):
+        t = int(toy_plain_logits(w, ids)[-1].argmax())
+        ids.append(t)
+        out.append(t)
+        if eos is not None and t == eos:
+            break
+    return out
+
+
+def _toy_generate(device, dtype, tmp_path, device_state, **options):
+    """The toy through the entry point: scheduler, portions of prompts, so few pages that requests are pushed
+    out and computed again (their state starts again from zero), steps issued ahead where the model allows."""
+    from nanohybrid_vlm_amd import LLM, SamplingParams
+    prompts = [rc.random_tokens(VOCAB, n, 60 + n) for n in (5, 19, 11, 26)]
+    results = {}
+    for what, pages in (("ample", 64), ("few pages", 17)):
+        folder = _toy_folder(tmp_path, device_state)
+        _, w = plain.read_model_folder(folder)
+        llm = LLM(folder, device=device, dtype=dtype, kvcache_block_size=4, num_kvcache_blocks=pages,
+                  max_num_batched_tokens=12, max_num_seqs=3, max_model_len=64, **options)
+        assert llm.config.eos == -1 and llm.config.max_model_len == 64      # the toy names no end token
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10), use_tqdm=False)
+        results[what] = [o["token_ids"] for o in outs]
+        if dtype == "float32":
+            assert results[what] == [_toy_greedy(w, p, 10) for p in prompts], what
+        if what == "few pages":
+            assert llm.scheduler.num_preemptions > 0, "the small cache was meant to force a request out"
+        stats = llm.get_memory_stats()
+        assert stats["live_requests"] == 0 and all(g["free_pages"] == g["pages"] for g in stats["groups"])
+        yield llm
+    assert results["ample"] == results["few pages"] or dtype != "float32"
+    # a configuration that names an end token: the engine takes it from the built model
+    folder = write_random_model(str(tmp_path / "toy_eos"), {"architectures": ["ToyForCausalLM"], "model_type": "toy",
+                                                            "device_state": device_state, "eos_token_id": 5}, seed=4)
+    llm = LLM(folder, device=device, dtype=dtype, kvcache_block_size=4, num_kvcache_blocks=32, max_model_len=64, **options)
+    assert llm.config.eos == 5
+
+
+@pytest.mark.parametrize("device_state", [False, True], ids=["state on the host", "state on the device"])
+def test_toy_generates_through_the_entry_point_on_emulated_kernels(toy_architecture, emulated_kernels, tmp_path, device_state):
+    for _ in _toy_generate("cpu", "float32", tmp_path, device_state):
+        pass
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("device_state", [False, True], ids=["state on the host", "state on the device"])
+def test_toy_generates_through_the_entry_point_on_gpu(toy_architecture, tmp_path, device_state, dtype):
+    for llm in _toy_generate("cuda:0", dtype, tmp_path, device_state):
+        stats = llm.get_memory_stats()
+        if device_state:
+            # per-request state keeps a model neither out of graphs nor out of steps issued ahead
+            assert stats["graphs_recorded"] and not stats["graphs_refused"], stats
+            assert llm.num_steps_ahead > 0
+        else:
+            assert not stats["graphs_recorded"] and llm.num_steps_ahead == 0
+
+
+@pytest.mark.gpu
+def test_toy_through_the_command_line(tmp_path):
+    """``--plugin`` imports the module that registers the toy; nothing in the package names it."""
+    env = dict(os.environ, PYTHONPATH=os.pathsep.join([os.path.join(REPO, "tests"), REPO, os.environ.get("PYTHONPATH", "")]))
+    toy.register()
+    try:
+        folder = _toy_folder(tmp_path, device_state=True)
+        _, w = plain.read_model_folder(folder)
+    finally:
+        toy.unregister()
+    proc = subprocess.run([sys.executable, "-m", "nanohybrid_vlm_amd", "generate", "--plugin", "toy_architecture",
+                           "--model", folder, "--dtype", "float32", "--prompt-ids", "5 17 3 60", "--prompt-ids", "9 8 7",
+                           "--output-tokens", "6", "--temperature", "0", "--block-size", "4", "--num-blocks", "32",
+                           "--max-model-len", "64", "--quiet"], cwd=REPO, env=env, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    out = json.loads(proc.stdout)
+    assert [o["token_ids"] for o in out] == [_toy_greedy(w, p, 6) for p in ([5, 17, 3, 60], [9, 8, 7])]
+    # random weights of a configuration given as a file, for an architecture the package does not know
+    cfg_file = tmp_path / "toy_config.json"
+    cfg_file.write_text(json.dumps({"architectures": ["ToyForCausalLM"], "model_type": "toy", "device_state": True}))
+    proc = subprocess.run([sys.executable, "-m", "nanohybrid_vlm_amd", "generate", "--plugin", "toy_architecture",
+                           "--random-weights", "3", "--config", str(cfg_file), "--prompt-ids", "1 2 3", "--output-tokens", "4",
+                           "--temperature", "0", "--block-size", "4", "--num-blocks", "32", "--max-model-len", "64", "--quiet"],
+                          cwd=REPO, env=env, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert len(json.loads(proc.stdout)[0]["token_ids"]) == 4
 
 
 def test_run_order_is_checked():
+    toy.register_parts()
     spec = toy_spec({})
-    _register_toy_parts()
     try:
         spec.run_order = [RunEntry(0), RunEntry(5)]
         with pytest.raises(ValueError, match="names layer 5"):
@@ -256,7 +180,7 @@ def test_run_order_is_checked():
         with pytest.raises(ValueError, match="earlier entry"):
             DecoderModel(spec)
     finally:
-        _unregister_toy_parts()
+        toy.unregister_parts()
     with pytest.raises(KeyError, match="unknown position encoding"):
         DecoderModel(toy_spec({}))
 

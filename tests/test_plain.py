@@ -170,3 +170,20 @@ def test_sampling_rule():
     assert (n >= 0).all() and abs(n.mean().item() - 1.0) < 0.1            # Exp(1) has mean 1
     assert torch.equal(n, plain.sample_noise(5, 2, 3, 1000))
     assert not torch.equal(n, plain.sample_noise(5, 2, 4, 1000))
+
+
+def test_noise_of_the_extreme_bit_patterns():
+    """The 24 bits' noise is the middle of their bucket of the Exp(1) distribution: the lowest noise is 3e-8, which
+    is what a true draw below 6e-8 is on average, and not 0 (or a floor of 1e-10, which would let an index of
+    chance 1e-9 win once in 2^24 draws); the share of patterns below x is 1 - exp(-x) to within one pattern."""
+    import math
+    import numpy as np
+    n = 1 << 24
+    assert math.isclose(plain.noise_of_bits(n - 1), 0.5 / n, rel_tol=1e-6)
+    assert math.isclose(plain.noise_of_bits(0), math.log(2 * n), rel_tol=1e-12)
+    values = np.array([plain.noise_of_bits(b) for b in list(range(n - 2000, n)) + list(range(0, n, 4099))])
+    assert (values > 2.9e-8).all() and np.isfinite(values).all()
+    for x in (1e-7, 1e-6, 1e-5, 1e-3, 0.5):
+        below = sum(1 for b in range(n - 1, n - 200, -1) if plain.noise_of_bits(b) < x) if x < 1e-5 else None
+        if below is not None:
+            assert abs(below / n - (1 - math.exp(-x))) <= 1.0 / n

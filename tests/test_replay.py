@@ -63,7 +63,7 @@ def _poisoned(runner):
     return runner
 
 
-def _run_all_modes(make_runner, folder, dtype, rounding_reference=False):
+def _run_all_modes(make_runner, folder, dtype, rounding_reference=False, stats=None):
     cfg, _ = plain.read_model_folder(folder)
     requests = _requests(cfg["vocab_size"])
     want = _rounding_reference(folder, requests) if rounding_reference else _plain_logits(folder, requests)
@@ -88,6 +88,9 @@ def _run_all_modes(make_runner, folder, dtype, rounding_reference=False):
         _check(results[mode], want, tol, f"{dtype} {mode}")
         assert not runner.cache.requests, "every request was ended"
         assert runner.cache.num_free_pages(0) == pages, "every page came back"
+        if stats is not None:
+            for key in stats:
+                stats[key] = sorted(set(stats[key]) | set(runner.get_memory_stats()[key]))
     return results
 
 
@@ -121,13 +124,23 @@ def test_replay_on_gpu(model_folders, name, dtype, graphs, tmp_path):
     folder = model_folders[name.split("_")[0]]
     if name.endswith("_sharp"):
         folder = sharpen(folder, str(tmp_path / "sharp"))
-    results = _run_all_modes(make, folder, dtype, rounding_reference=(dtype == "bfloat16" and name.endswith("_sharp")))
-    if dtype == "float32":
-        # in 32-bit the ways of cutting agree with each other far more closely than with the plain implementation
-        for mode in ("tail", "portions", "mixed"):
-            for rid in results["whole"]:
+    runner_stats = {"graphs_recorded": [], "graphs_refused": []}
+    results = _run_all_modes(make, folder, dtype, rounding_reference=(dtype == "bfloat16" and name.endswith("_sharp")),
+                             stats=runner_stats)
+    if graphs:
+        assert runner_stats["graphs_recorded"] and not runner_stats["graphs_refused"], runner_stats
+    for mode in ("tail", "portions", "mixed"):
+        for rid in results["whole"]:
+            if dtype == "float32":
+                # in 32-bit every sum has one order, whatever the batch: the ways of cutting agree bit for bit
+                assert torch.equal(results[mode][rid], results["whole"][rid]), \
+                    f"float32 {mode} against whole: request {rid}: {max_abs_diff(results[mode][rid], results['whole'][rid]):.3e}"
+            else:
+                # in bfloat16 all ways store the same keys and values (one kernel writes them) and round the same
+                # tensors; what differs is the attention kernel (prompt portions or single tokens) and the order of
+                # sums: far less than the distance to the plain implementation, also where the scores are sharpened
                 d = max_abs_diff(results[mode][rid], results["whole"][rid])
-                assert d <= 2e-6, f"float32 {mode} against whole: request {rid}: {d:.3e}"
+                assert d <= 0.5 * TOLERANCE["bfloat16"], f"bfloat16 {mode} against whole: request {rid}: {d:.3e}"
 
 
 @pytest.mark.gpu
@@ -247,27 +260,95 @@ def _trace_run(folder, dtype, steps, out_dir, max_tokens, extra=()):
     return proc
 
 
-@pytest.mark.gpu
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run_program(model_folders, dtype, tmp_path):
-    """The program itself, as a user starts it: mixed trace, pool made for the trace's peak, files compared."""
-    folder = model_folders["B"]
-    cfg, w = plain.read_model_folder(folder)
-    requests = {f"r{i}": rc.random_tokens(cfg["vocab_size"], n, 7 + i) for i, n in enumerate([70, 130, 9, 64, 65, 100])}
-    steps = rc.mixed(requests)
-    out_dir = str(tmp_path / "out")
-    _trace_run(folder, dtype, steps, out_dir, rc.peak_tokens(steps, 64))
-    want = {rid: plain.logits(cfg, w, toks) for rid, toks in requests.items()}
-    fed = {rid: 0 for rid in requests}
-    V = cfg["vocab_size"]
+def _renamed(steps, suffix, first_step):
+    """The same trace with other request names and step numbers, so that several traces can follow each other in
+    one run of the program."""
+    out = []
+    for i, st in enumerate(steps):
+        out.append({"step": first_step + i, "entries": [dict(e, id=e["id"] + suffix) for e in st["entries"]],
+                    "end": [r + suffix for r in st["end"]]})
+    return out
+
+
+def _logits_from_files(out_dir, steps, vocab):
+    """Per request the logits of all its tokens, from the program's <step>.f32 files."""
+    parts = {}
     for st in steps:
-        data = np.fromfile(os.path.join(out_dir, f"{st['step']}.f32"), dtype="<f4").reshape(-1, V)
+        wanted = sum(len(e["want"]) for e in st["entries"])
+        path = os.path.join(out_dir, f"{st['step']}.f32")
+        if not wanted:
+            assert not os.path.exists(path)
+            continue
+        data = np.fromfile(path, dtype="<f4").reshape(-1, vocab)
+        assert data.shape[0] == wanted
         row = 0
         for e in st["entries"]:
-            n = len(e["tokens"])
-            ref = want[e["id"]][fed[e["id"]]:fed[e["id"]] + n]
-            d = max_abs_diff(torch.from_numpy(data[row:row + n].copy()), ref)
-            assert d <= TOLERANCE[dtype], f"step {st['step']} request {e['id']}: {d:.3e}"
-            fed[e["id"]] += n
-            row += n
-        assert row == data.shape[0]
+            n = len(e["want"])
+            if n:
+                parts.setdefault(e["id"], []).append(torch.from_numpy(data[row:row + n].copy()))
+                row += n
+    return {rid: torch.cat(p) for rid, p in parts.items()}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_trace_run_program_in_the_four_ways(model_folders, name, dtype, tmp_path):
+    """The program itself, as a user starts it, fed the same requests whole, with the last 32 tokens one by one, in
+    portions of changing size and mixed on few pages (one run: the four traces follow each other, and the pool is
+    made for the largest peak). Every position against the plain implementation; in float32 the four ways agree
+    bit for bit."""
+    folder = model_folders[name]
+    cfg, w = plain.read_model_folder(folder)
+    requests = {f"r{i}": rc.random_tokens(cfg["vocab_size"], n, 7 + i) for i, n in enumerate([70, 130, 9, 64, 65, 100])}
+    ways = {"whole": rc.whole(requests), "tail": rc.tail_decoded(requests), "portions": rc.portions(requests),
+            "mixed": rc.mixed(requests)}
+    steps, first = [], 0
+    for way, trace in ways.items():
+        ways[way] = _renamed(trace, "_" + way, first)
+        steps += ways[way]
+        first += len(trace)
+    out_dir = str(tmp_path / "out")
+    _trace_run(folder, dtype, steps, out_dir, max(rc.peak_tokens(t, 64) for t in ways.values()))
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in requests.items()}
+    got = _logits_from_files(out_dir, steps, cfg["vocab_size"])
+    for way in ways:
+        for rid in requests:
+            d = max_abs_diff(got[f"{rid}_{way}"], want[rid])
+            assert d <= TOLERANCE[dtype], f"{way}: request {rid}: {d:.3e}; " + first_difference(got[f"{rid}_{way}"], want[rid], TOLERANCE[dtype])
+            if dtype == "float32":
+                assert torch.equal(got[f"{rid}_{way}"], got[f"{rid}_whole"]), f"float32: {way} differs from whole for {rid}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("page", [256, 48])
+def test_trace_run_program_with_other_page_sizes(model_folders, page, tmp_path):
+    """Pages of 256 tokens (the engine's default) and of 48 (neither a divisor nor a multiple of 64): the pool is made
+    from --max-tokens, counted in units of 64 as a caller counts it, and the mixed trace fits and is right."""
+    folder = model_folders["D"]
+    cfg, w = plain.read_model_folder(folder)
+    requests = {f"r{i}": rc.random_tokens(cfg["vocab_size"], n, 70 + i) for i, n in enumerate([300, 70, 513, 64, 129, 40])}
+    steps = rc.mixed(requests, sizes=(100, 7, 64, 2, 129, 33))
+    out_dir = str(tmp_path / "out")
+    _trace_run(folder, "bfloat16", steps, out_dir, rc.peak_tokens(steps, 64), extra=("--page-size", str(page)))
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in requests.items()}
+    got = _logits_from_files(out_dir, steps, cfg["vocab_size"])
+    tol = tolerance_for("bfloat16", want)
+    for rid in requests:
+        d = max_abs_diff(got[rid], want[rid])
+        assert d <= tol, f"pages of {page}: request {rid}: {d:.3e}"
+
+
+def test_pool_of_a_replay():
+    from nanohybrid_vlm_amd.engine.replay import pages_for
+    assert pages_for(640, 64) == 10 and pages_for(640, 8) == 80 and pages_for(640, 1) == 640
+    # four requests of 65 tokens are counted as 4 x 128 = 512; with pages of 256 each needs one page, of 48 two
+    assert pages_for(512, 256) >= 4 and pages_for(512, 48) >= 8
+    # the worst case for pages of 256: four requests of 257..320 tokens, counted as 4 x 320
+    assert pages_for(4 * 320, 256) >= 8
+    for page in (3, 48, 100, 256, 1000):
+        for lengths in ([1, 1, 1, 1], [64, 65, 129, 300], [257, 320, 513, 1], [1000, 999, 63, 64]):
+            counted = sum(-(-n // 64) * 64 for n in lengths)
+            assert pages_for(counted, page) >= sum(-(-n // page) for n in lengths), (page, lengths)
+
+
