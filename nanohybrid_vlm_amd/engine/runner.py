@@ -455,13 +455,14 @@ class ModelRunner:
         g = self._graphs.get(next(b for b in self.graph_buckets if b >= len(request_ids)))
         if g is None or g["graph"] is None:
             return False
-        longest = max(256, max(self.cache.num_tokens(r) for r in request_ids) + 1)
+        real = max(self.cache.num_tokens(r) for r in request_ids) + 1
+        longest = max(256, real)                       # (short contexts share one graph, as in _graph_step)
         need = [0] * len(self.cache.groups)
         for r in request_ids:
             for gi, n in enumerate(self.cache.pages_needed(r, self.cache.num_tokens(r) + 1)):
                 need[gi] += n
-        return (g["planned"] // 2 < longest <= g["planned"] + g["planned"] // 2 and longest <= self.max_model_len
-                and longest <= self.max_position and all(n <= self.cache.num_free_pages(gi) for gi, n in enumerate(need)))
+        return (g["planned"] // 2 < longest <= g["planned"] + g["planned"] // 2 and real <= self.max_model_len
+                and real <= self.max_position and all(n <= self.cache.num_free_pages(gi) for gi, n in enumerate(need)))
 
     @torch.no_grad()
     def step_ahead(self, request_ids: list, tokens: torch.Tensor) -> dict:

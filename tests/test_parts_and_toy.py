@@ -32,7 +32,7 @@ def toy_architecture():
 
 def _toy_folder(tmp_path, device_state=False, **keys):
     cfg = {"architectures": ["ToyForCausalLM"], "model_type": "toy", "device_state": device_state, **keys}
-    return write_random_model(str(tmp_path / f"toy{int(device_state)}"), cfg, seed=4)
+    return write_random_model(str(tmp_path / f"toy{int(device_state)}{int(bool(keys.get('no_window')))}"), cfg, seed=4)
 
 
 def _toy_check(device, dtype, tol, tmp_path, device_state=False, graphs=False):
@@ -78,10 +78,10 @@ def test_toy_architecture_on_gpu(toy_architecture, dtype, tol, tmp_path, device_
     _toy_check("cuda:0", dtype, tol, tmp_path, device_state, graphs)
 
 
-def _toy_greedy(w, prompt, n, eos=None):
+def _toy_greedy(w, prompt, n, eos=None, no_window=False):
     ids, out = list(prompt), []
     for _ in range(n):
-        t = int(toy_plain_logits(w, ids)[-1].argmax())
+        t = int(toy_plain_logits(w, ids, no_window)[-1].argmax())
         ids.append(t)
         out.append(t)
         if eos is not None and t == eos:
@@ -89,22 +89,23 @@ def _toy_greedy(w, prompt, n, eos=None):
     return out
 
 
-def _toy_generate(device, dtype, tmp_path, device_state, **options):
+def _toy_generate(device, dtype, tmp_path, device_state, no_window=False, **options):
     """The toy through the entry point: scheduler, portions of prompts, so few pages that requests are pushed
     out and computed again (their state starts again from zero), steps issued ahead where the model allows."""
     from nanohybrid_vlm_amd import LLM, SamplingParams
     prompts = [rc.random_tokens(VOCAB, n, 60 + n) for n in (5, 19, 11, 26)]
     results = {}
-    for what, pages in (("ample", 64), ("few pages", 17)):
-        folder = _toy_folder(tmp_path, device_state)
+    for what, pages in (("ample", 64), ("few pages", 13)):
+        folder = _toy_folder(tmp_path, device_state, no_window=no_window)
         _, w = plain.read_model_folder(folder)
+        # (no prompt is ever overdue: what is pushed out is pushed out for pages, on a fast machine and a slow one)
         llm = LLM(folder, device=device, dtype=dtype, kvcache_block_size=4, num_kvcache_blocks=pages,
-                  max_num_batched_tokens=12, max_num_seqs=3, max_model_len=64, **options)
+                  max_num_batched_tokens=12, max_num_seqs=3, max_model_len=64, max_prefill_wait_ms=1e9, **options)
         assert llm.config.eos == -1 and llm.config.max_model_len == 64      # the toy names no end token
         outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10), use_tqdm=False)
         results[what] = [o["token_ids"] for o in outs]
         if dtype == "float32":
-            assert results[what] == [_toy_greedy(w, p, 10) for p in prompts], what
+            assert results[what] == [_toy_greedy(w, p, 10, no_window=no_window) for p in prompts], what
         if what == "few pages":
             assert llm.scheduler.num_preemptions > 0, "the small cache was meant to force a request out"
         stats = llm.get_memory_stats()
@@ -126,14 +127,16 @@ def test_toy_generates_through_the_entry_point_on_emulated_kernels(toy_architect
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("device_state", [False, True], ids=["state on the host", "state on the device"])
-def test_toy_generates_through_the_entry_point_on_gpu(toy_architecture, tmp_path, device_state, dtype):
-    for llm in _toy_generate("cuda:0", dtype, tmp_path, device_state):
+@pytest.mark.parametrize("device_state,no_window", [(False, False), (True, False), (True, True)],
+                         ids=["state on the host", "state on the device", "state on the device, no window"])
+def test_toy_generates_through_the_entry_point_on_gpu(toy_architecture, tmp_path, device_state, no_window, dtype):
+    for llm in _toy_generate("cuda:0", dtype, tmp_path, device_state, no_window):
         stats = llm.get_memory_stats()
         if device_state:
-            # per-request state keeps a model neither out of graphs nor out of steps issued ahead
+            # per-request state keeps a model neither out of graphs nor out of steps issued ahead (a step issued
+            # ahead may have to be taken back, which a window's pages, given back as it moves, do not allow)
             assert stats["graphs_recorded"] and not stats["graphs_refused"], stats
-            assert llm.num_steps_ahead > 0
+            assert (llm.num_steps_ahead > 0) == no_window
         else:
             assert not stats["graphs_recorded"] and llm.num_steps_ahead == 0
 

@@ -9,8 +9,10 @@ entry's cache; and its plain whole-sequence computation.
 Importing this module registers the parts and the architecture (so the command line can
 take it as ``--plugin toy_architecture``); ``unregister()`` takes them out again.
 config.json of a toy model: {"architectures": ["ToyForCausalLM"], "model_type": "toy",
-"device_state": bool, "eos_token_id": int or absent}.
+"device_state": bool, "no_window": bool, "eos_token_id": int or absent}.
 """
+import math
+
 import torch
 
 import plain_qwen3 as plain
@@ -72,14 +74,19 @@ class DecayingSumOnDevice(DecayingSum):
         first_row = batch.cu_seqlens_q[:-1].long()                      # [B] row of every request's first token
         last_row = batch.cu_seqlens_q[1:].long() - 1
         slots = step.state_slots.long()
-        y = x.to(torch.float64) * torch.pow(self.decay, -pos)[:, None]
+        log_decay = math.log(self.decay)
+
+        def power(exponent):                                            # decay^exponent, from device tensors only
+            return torch.exp(exponent * log_decay)
+
+        y = x.to(torch.float64) * power(-pos)[:, None]
         c = torch.cumsum(y, dim=0)
         within = c - (c[first_row] - y[first_row])[req]                # sums that start at the request's first row
         first_pos = pos[first_row]
         before = torch.where((first_pos == 0)[:, None], torch.zeros_like(pool[slots], dtype=torch.float64),
                              pool[slots].to(torch.float64))
-        carried = before * torch.pow(self.decay, 1.0 - first_pos)[:, None]
-        s = (within + carried[req]) * torch.pow(self.decay, pos)[:, None]
+        carried = before * power(1.0 - first_pos)[:, None]
+        s = (within + carried[req]) * power(pos)[:, None]
         pool[slots] = s[last_row].to(pool.dtype)
         return (s.to(torch.float32) @ self.weight.float().T).to(x.dtype)
 
@@ -89,8 +96,11 @@ class RoutedFeedForward(Part):
     the expert it rates highest (the experts are the package's own gated feed-forwards, built through the
     registry) and the result is weighted with that expert's probability."""
 
-    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, on_device: bool = False):
         self.hidden_size = hidden_size
+        # False: the rows of every expert are looked up on the host and only those go through it (a step with
+        # this cannot be recorded); True: every expert sees every row and a mask keeps the chosen ones
+        self.recordable = on_device
         self.experts = [FEED_FORWARDS.build({"kind": "swiglu", "hidden_size": hidden_size,
                                              "intermediate_size": intermediate_size}) for _ in range(num_experts)]
 
@@ -107,6 +117,11 @@ class RoutedFeedForward(Part):
         prob = torch.softmax(x.float() @ self.router.float().T, dim=-1)
         best = prob.argmax(dim=-1)
         out = torch.zeros_like(x)
+        if self.recordable:
+            for e, expert in enumerate(self.experts):
+                y = expert.forward(x, step).float() * prob[:, e:e + 1]
+                out = torch.where((best == e)[:, None], y.to(x.dtype), out)
+            return out
         for e, expert in enumerate(self.experts):
             rows = (best == e).nonzero().flatten()
             if rows.numel():
@@ -139,11 +154,12 @@ def toy_spec(cfg: dict) -> ModelSpec:
     def attention(window):
         return {"kind": "gqa_attention", "hidden_size": H, "num_heads": HEADS, "num_kv_heads": KV, "head_dim": D,
                 "scale": D ** -0.5, "qk_norm_eps": 1e-5, "qkv_bias": False, "window": window}
-    routed = {"kind": "toy_routed", "hidden_size": H, "intermediate_size": EXPERT_INTER, "num_experts": EXPERTS}
+    routed = {"kind": "toy_routed", "hidden_size": H, "intermediate_size": EXPERT_INTER, "num_experts": EXPERTS,
+              "on_device": bool(cfg.get("device_state"))}
     layers = [
         LayerSpec(mixer=attention(None), feed_forward=ff, norm=norm),
         LayerSpec(mixer={"kind": state_mixer, "hidden_size": H, "decay": DECAY}, feed_forward=routed, norm=norm),
-        LayerSpec(mixer=attention(WINDOW), feed_forward=ff, norm=norm, position="linear"),
+        LayerSpec(mixer=attention(None if cfg.get("no_window") else WINDOW), feed_forward=ff, norm=norm, position="linear"),
     ]
     # layer 0 runs twice (two caches); the last entry runs layer 2 again on the keys and values of entry 2
     order = [RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(2, cache=2)]
@@ -165,15 +181,16 @@ def toy_turn(x, pos):
     return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., TOY_ROT:]), dim=-1)
 
 
-def toy_plain_logits(w, toks):
+def toy_plain_logits(w, toks, no_window=False):
     """Whole sequence, no cache, from the plain functions."""
+    window_of_layer_2 = None if no_window else WINDOW
     T = len(toks)
     pos = torch.arange(T)
     r = w["embed.weight"][toks]
     kept = {}
 
     def attention(x, p, window, entry, lender=None):
-        turn = toy_turn if window else (lambda t, at: plain.apply_rope(t, at, 1000.0))   # the windowed layer has the toy angles
+        turn = toy_turn if p.startswith("layers.2.") else (lambda t, at: plain.apply_rope(t, at, 1000.0))   # layer 2 has the toy angles
         qkv = x @ w[p + "mixer.qkv.weight"].T
         q = plain.rms_norm(qkv[:, :HEADS * D].view(T, HEADS, D), w[p + "mixer.q_norm.weight"], 1e-5)
         if lender is None:
@@ -207,7 +224,7 @@ def toy_plain_logits(w, toks):
         if layer == 1:
             r = r + decaying_sum(x, p)
         else:
-            r = r + attention(x, p, WINDOW if layer == 2 else None, entry, lender)
+            r = r + attention(x, p, window_of_layer_2 if layer == 2 else None, entry, lender)
         x = plain.rms_norm(r, w[p + "feed_forward_norm.weight"], 1e-5)
         if layer == 1:
             r = r + routed(x, p)
