@@ -31,7 +31,9 @@
 // wave on splits of 256), nothing at 1, 8 and 64 requests or at 8,192 keys; inside the model's decoding step the same
 // choice took 2 to 5 % more time at 24, 32 and 48 requests.)
 #include "nhv_common.h"
+#include "nhv_no_alloc.h"
 #include <math.h>
+#include <mutex>
 
 #ifndef NHV_HEAD_DIM
 #error "compile with -DNHV_HEAD_DIM=<head size>"
@@ -321,26 +323,17 @@ __global__ __launch_bounds__(64 * W) void merge_splits_kernel(const float* __res
 
 extern "C" int nhv_decode_attention_head_dim() { return D; }
 
-// part_o: float [T, Hq, n_splits, D]; part_ml: float [T, Hq, n_splits, 2]; n_splits * split_len must cover
-// every context length of the batch (max_context_len).
-extern "C" int nhv_decode_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out, void* part_o,
-                                         void* part_ml, const void* token_req, const void* positions,
-                                         const void* block_tables, int max_blocks, int T, int Hq, int Hkv, int page_size,
-                                         float scale, int window, int split_len, int n_splits, void* stream) {
-  NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && page_size > 0 && max_blocks > 0, "decode attention: bad sizes");
+// Checks and launches shared by the two entry points.
+static int launch_decode_attention(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_o,
+                                   float* part_ml, const void* token_req, const void* positions,
+                                   const void* block_tables, int max_blocks, int T, int Hq, int Hkv, int page_size,
+                                   float scale, int window, int split_len, int n_splits, hipStream_t s) {
   int page_shift = -1;
   for (int b = 0; b < 31; ++b)
     if (page_size == (1 << b)) page_shift = b;
-  NHV_REQUIRE(Hq % Hkv == 0, "decode attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
-  const int G = Hq / Hkv;
-  NHV_REQUIRE(G <= 16, "decode attention: %d query heads per key head are beyond this kernel's limit of 16", G);
-  NHV_REQUIRE(split_len > 0 && split_len % RK == 0, "decode attention: split length %d must be a multiple of %d", split_len, RK);
-  NHV_REQUIRE(n_splits > 0 && n_splits <= 65535 && Hkv <= 65535 && T <= 65535, "decode attention: grid too large");
-  NHV_REQUIRE(window >= 0, "decode attention: negative window");
-  hipStream_t s = (hipStream_t)stream;
   dim3 grid(Hkv, T, n_splits);
   hipLaunchKernelGGL(decode_attention_kernel, grid, dim3(64), 0, s, (const bf16_t*)q, (const bf16_t*)k_cache,
-                     (const bf16_t*)v_cache, (float*)part_o, (float*)part_ml, (const int*)token_req,
+                     (const bf16_t*)v_cache, part_o, part_ml, (const int*)token_req,
                      (const int*)positions, (const int*)block_tables, max_blocks, Hq, Hkv, page_size, page_shift,
                      scale * 1.4426950408889634f, window, split_len, n_splits);
   NHV_LAUNCH_CHECK("decode_attention");
@@ -354,4 +347,78 @@ extern "C" int nhv_decode_attention_bf16(const void* q, const void* k_cache, con
                        (const float*)part_ml, (bf16_t*)out, (const int*)positions, window, split_len, n_splits, Hq);
   NHV_LAUNCH_CHECK("merge_splits");
   return 0;
+}
+
+static int check_decode_attention(int max_blocks, int T, int Hq, int Hkv, int page_size, int window, int split_len,
+                                  int n_splits) {
+  NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && page_size > 0 && max_blocks > 0, "decode attention: bad sizes");
+  NHV_REQUIRE(Hq % Hkv == 0, "decode attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
+  const int G = Hq / Hkv;
+  NHV_REQUIRE(G <= 16, "decode attention: %d query heads per key head are beyond this kernel's limit of 16", G);
+  NHV_REQUIRE(split_len > 0 && split_len % RK == 0, "decode attention: split length %d must be a multiple of %d", split_len, RK);
+  NHV_REQUIRE(n_splits > 0 && n_splits <= 65535 && Hkv <= 65535 && T <= 65535, "decode attention: grid too large");
+  NHV_REQUIRE(window >= 0, "decode attention: negative window");
+  return 0;
+}
+
+// part_o: float [T, Hq, n_splits, D]; part_ml: float [T, Hq, n_splits, 2]; n_splits * split_len must cover
+// every context length of the batch (max_context_len).
+extern "C" int nhv_decode_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out, void* part_o,
+                                         void* part_ml, const void* token_req, const void* positions,
+                                         const void* block_tables, int max_blocks, int T, int Hq, int Hkv, int page_size,
+                                         float scale, int window, int split_len, int n_splits, void* stream) {
+  if (check_decode_attention(max_blocks, T, Hq, Hkv, page_size, window, split_len, n_splits)) return 1;
+  return launch_decode_attention(q, k_cache, v_cache, out, (float*)part_o, (float*)part_ml, token_req, positions,
+                                 block_tables, max_blocks, T, Hq, Hkv, page_size, scale, window, split_len, n_splits,
+                                 (hipStream_t)stream);
+}
+
+// ---- the entry point that allocates nothing (nhv_no_alloc.h) ----
+// The splits' partial results of a call: [T, Hq, n_splits, D] floats, then [T, Hq, n_splits, 2]. Part of the
+// library's device image: every GPU that loads the library holds its own copy at its own address.
+constexpr size_t SCRATCH_FLOATS = NHV_NO_ALLOC_SCRATCH_BYTES / sizeof(float);
+static __device__ __align__(256) float scratch[SCRATCH_FLOATS];
+
+// In host code the array's name stands for a host-side handle, not for device memory: each device's address
+// is asked for once, with that device current, and kept.
+constexpr int MAX_DEVICES = 64;
+static float* scratch_of_device[MAX_DEVICES] = {};
+static std::mutex scratch_lock;
+
+static int scratch_address(float** ptr) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  NHV_REQUIRE(e == hipSuccess, "decode attention (no alloc): hipGetDevice failed: %s", hipGetErrorString(e));
+  NHV_REQUIRE(device >= 0 && device < MAX_DEVICES, "decode attention (no alloc): device %d is beyond the %d this library keeps track of",
+              device, MAX_DEVICES);
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_of_device[device] == nullptr) {
+    void* address = nullptr;
+    e = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+    NHV_REQUIRE(e == hipSuccess && address != nullptr, "decode attention (no alloc): hipGetSymbolAddress failed on device %d: %s",
+                device, hipGetErrorString(e));
+    scratch_of_device[device] = (float*)address;
+  }
+  *ptr = scratch_of_device[device];
+  return 0;
+}
+
+extern "C" size_t nhv_decode_attention_no_alloc_limit() { return NHV_NO_ALLOC_SCRATCH_BYTES; }
+
+extern "C" int nhv_decode_attention_bf16_no_alloc(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                                  const void* token_req, const void* positions,
+                                                  const void* block_tables, int max_blocks, int T, int Hq, int Hkv,
+                                                  int page_size, float scale, int window, int split_len, int n_splits,
+                                                  void* stream) {
+  if (check_decode_attention(max_blocks, T, Hq, Hkv, page_size, window, split_len, n_splits)) return 1;
+  const size_t items = (size_t)T * Hq * n_splits;
+  NHV_REQUIRE(items * (D + 2) <= SCRATCH_FLOATS,
+              "decode attention (no alloc): %d tokens x %d heads x %d splits need %zu bytes of scratch, the library holds %zu",
+              T, Hq, n_splits, items * (D + 2) * sizeof(float), (size_t)NHV_NO_ALLOC_SCRATCH_BYTES);
+  float* base = nullptr;
+  if (scratch_address(&base)) return 1;
+  // a call reads only the entries it has written (the merge looks at the splits that hold a visible key, and
+  // those are the splits that write): nothing has to be cleared
+  return launch_decode_attention(q, k_cache, v_cache, out, base, base + items * D, token_req, positions, block_tables,
+                                 max_blocks, T, Hq, Hkv, page_size, scale, window, split_len, n_splits, (hipStream_t)stream);
 }
