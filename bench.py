@@ -1,16 +1,20 @@
-"""Decode and prefill throughput of the Qwen3-8B shape with random bfloat16 weights
-on one MI355X, through the engine's own entry point (scheduler, step function,
-cache, kernels, sampler).
+"""Decode and prefill throughput of the Qwen3 shapes with random bfloat16 weights on one MI355X, through the
+engine's own entry point (scheduler, step function, cache, kernels, sampler).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--shape 8b|14b|32b] [--layers L]
 
-A step is one decode step of the whole batch. Each request is a 2,048-token prompt
-of random ids followed by generated tokens; W steps run untimed, then exactly K
-steps are timed between two synchronisations. One JSON line is printed: ``value``
-is decoded tokens a second; ``prefill`` is one 2,048-token prompt; ``roofline``
-compares the decode step with the time to read what it must read (all weights it
-uses once, and the cache of the live requests) at 8 TB/s; ``points`` holds decoding
-at batch 1 and 64.
+Default (``--shape 8b``): a step is one decode step of the whole batch. Each request is a 2,048-token prompt of
+random ids followed by generated tokens; W steps run untimed, then exactly K steps are timed between two
+synchronisations. One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` is one 2,048-token
+prompt; ``roofline`` compares the decode step with the time to read what it must read (all weights it uses once, and
+the cache of the live requests) at 8 TB/s, and ``measured`` gives the same fractions against what this GPU was
+measured to give (a kernel that only reads; the vendor library's large bfloat16 product); ``points`` holds
+decoding at batch 1 and 64; ``step_ms`` the timed steps' median and 95th percentile.
+
+``--shape 14b``: 32 requests with prompt lengths uniform in [128, 4096] and 128 generated tokens each, all queued at
+once, prompts fed in portions of 2,048 tokens beside the decoding requests (continuous batching).
+``--shape 32b``: 16 requests of 8,192 prompt tokens and 256 generated tokens, the cache sized from free memory.
+For these two ``value`` is generated tokens a second over the whole run, prompts included; a step is an engine step.
 """
 import argparse
 import json
@@ -26,20 +30,32 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=192)
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=None, help="requests decoding side by side (8b: 8, 14b: 32, 32b: 16)")
     ap.add_argument("--shape", default="8b")
+    ap.add_argument("--workload", default="auto", choices=("auto", "points", "serving"),
+                    help="points: decode at a fixed batch after equal prompts (8b by default); serving: the 14b / 32b workloads")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (same layer sizes)")
-    ap.add_argument("--prompt-tokens", type=int, default=2048)
-    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prompt-tokens", type=int, default=None, help="8b: 2048; 32b: 8192; 14b: the longest prompt, 4096")
+    ap.add_argument("--output-tokens", type=int, default=None, help="14b: 128; 32b: 256")
+    ap.add_argument("--context", type=int, default=None, help="max_model_len (8b: 4096)")
     ap.add_argument("--block-size", type=int, default=256)
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 runs")
+    ap.add_argument("--no-measured-peaks", action="store_true", help="skip the measurement of what this GPU gives")
     ap.add_argument("--eager", action="store_true", help="no HIP graphs")
     ap.add_argument("--max-graph-batch", type=int, default=None, help="largest decode batch that replays a graph")
+    ap.add_argument("--gemm-choices", default=None, help="JSON file of matrix-product choices to follow (and to write if absent)")
     return ap.parse_args()
 
 
-def build_llm(args, max_seqs):
+def percentile(values, q):
+    values = sorted(values)
+    k = (len(values) - 1) * q
+    lo, hi = int(k), min(int(k) + 1, len(values) - 1)
+    return values[lo] + (values[hi] - values[lo]) * (k - lo)
+
+
+def build_llm(args, max_seqs, **options):
     from nanohybrid_vlm_amd import LLM
     from nanohybrid_vlm_amd.config.registry import named_shapes
 
@@ -47,12 +63,9 @@ def build_llm(args, max_seqs):
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
-    pages_per_seq = -(-args.context // args.block_size)
-    llm = LLM(raw, random_weights=0, dtype=args.dtype,
-              kvcache_block_size=args.block_size, num_kvcache_blocks=max_seqs * pages_per_seq + 1,
-              max_num_seqs=max_seqs, max_num_batched_tokens=max(2048, max_seqs), max_model_len=args.context,
-              scheduler_policy="prefill_first",     # while prompts are fed nothing decodes, so all requests decode in step
-              enforce_eager=args.eager, **({"max_graph_batch": args.max_graph_batch} if args.max_graph_batch else {}))
+    llm = LLM(raw, random_weights=0, dtype=args.dtype, kvcache_block_size=args.block_size, max_num_seqs=max_seqs,
+              enforce_eager=args.eager, gemm_choices=args.gemm_choices,
+              **({"max_graph_batch": args.max_graph_batch} if args.max_graph_batch else {}), **options)
     return llm, llm.runner.cfg, full_layers
 
 
@@ -74,7 +87,8 @@ def random_prompts(n, length, vocab, seed):
 
 
 def run_decode(llm, cfg, batch, prompt_tokens, steps, warmup, seed):
-    """Prefills ``batch`` prompts, then times ``steps`` decode steps. Returns (seconds, mean context in the timed steps)."""
+    """Prefills ``batch`` prompts, then times ``steps`` decode steps. Returns (seconds, mean context in the timed
+    steps, the steps' host times in ms)."""
     import torch
     from nanohybrid_vlm_amd import SamplingParams
 
@@ -86,16 +100,21 @@ def run_decode(llm, cfg, batch, prompt_tokens, steps, warmup, seed):
     for _ in range(warmup):
         llm.step()
     torch.cuda.synchronize()
+    step_ms = []
     t0 = time.perf_counter()
+    last = t0
     for _ in range(steps):
         _, stats = llm.step()
         assert stats.num_decode_tokens == batch and stats.num_prefill_tokens == 0
+        now = time.perf_counter()
+        step_ms.append((now - last) * 1e3)
+        last = now
     torch.cuda.synchronize()
     seconds = time.perf_counter() - t0
     while not llm.is_finished():
         llm.step()
     mean_context = prompt_tokens + warmup + (steps + 1) / 2.0
-    return seconds, mean_context
+    return seconds, mean_context, step_ms
 
 
 def run_prefill(llm, cfg, prompt_tokens, reps=3):
@@ -118,63 +137,178 @@ def run_prefill(llm, cfg, prompt_tokens, reps=3):
     return best
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
-        return 2
+def config_of(args, cfg, full_layers, **more):
+    """Every size, flat (at most 20 keys)."""
+    out = {
+        "model": f"Qwen3-{args.shape} shape", "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers,
+        "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+        "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+        "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps, "tied_head": cfg.tie_word_embeddings,
+        "kv_block": args.block_size, "parallelism": "single GPU", "graphs": not args.eager,
+    }
+    out.update(more)
+    assert len(out) <= 20
+    return out
+
+
+def measured_peaks(args):
+    if args.no_measured_peaks:
+        return None
+    from nanohybrid_vlm_amd.native import ops
+    peaks = ops.measured_peaks()
+    return {"hbm_read_GBs": round(peaks["hbm_read_GBs"], 1), "gemm_bf16_TFLOPs": round(peaks["gemm_bf16_TFLOPs"], 1)}
+
+
+def bench_decode_points(args):
+    """The headline measurement: decode at a fixed batch after equal prompts, a 2,048-token prefill, batch 1 and 64."""
     import torch
 
+    batch = args.batch or 8
+    T = args.prompt_tokens or 2048
+    context = args.context or 4096
     itemsize = 2 if args.dtype == "bfloat16" else 4
     dname = "bf16" if args.dtype == "bfloat16" else "fp32"
-    max_seqs = max(args.batch, 1 if args.no_points else 64)
-    llm, cfg, full_layers = build_llm(args, max_seqs)
+    max_seqs = max(batch, 1 if args.no_points else 64)
+    pages_per_seq = -(-context // args.block_size)
+    llm, cfg, full_layers = build_llm(args, max_seqs, num_kvcache_blocks=max_seqs * pages_per_seq + 1,
+                                      max_num_batched_tokens=max(2048, max_seqs), max_model_len=context,
+                                      scheduler_policy="prefill_first")   # while prompts are fed nothing decodes, so all requests decode in step
     weight_bytes, kv_per_token, matrix_flops = model_bytes_and_flops(cfg, itemsize)
+    peaks = measured_peaks(args)
 
-    # prefill of one prompt
-    T = args.prompt_tokens
     pre_s = run_prefill(llm, cfg, T)
     attn_flops = 2 * 2 * cfg.num_hidden_layers * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2)
     pre_flops = matrix_flops * T + attn_flops + 2 * cfg.vocab_size * cfg.hidden_size
     prefill = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
                "frac": round(pre_flops / pre_s / PEAK_FLOPS[dname], 4)}
 
-    def decode_point(batch, steps, warmup, seed):
-        s, ctx = run_decode(llm, cfg, batch, T, steps, warmup, seed)
+    def decode_point(b, steps, warmup, seed):
+        s, ctx, step_ms = run_decode(llm, cfg, b, T, steps, warmup, seed)
         ms = s / steps * 1e3
-        step_bytes = weight_bytes + batch * ctx * kv_per_token
-        return batch * steps / s, ms, step_bytes / (ms * 1e-3) / 1e9
+        step_bytes = weight_bytes + b * ctx * kv_per_token
+        return b * steps / s, ms, step_bytes / (ms * 1e-3) / 1e9, step_ms
 
-    value, ms_per_step, achieved = decode_point(args.batch, args.steps, args.warmup, 1)
+    value, ms_per_step, achieved, step_ms = decode_point(batch, args.steps, args.warmup, 1)
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            if b == args.batch:
+            if b == batch:
                 points[f"decode_b{b}"] = round(value, 1)
                 continue
-            v, _, _ = decode_point(b, min(args.steps, 128), min(args.warmup, 8), 10 + b)
+            v, _, _, _ = decode_point(b, min(args.steps, 128), min(args.warmup, 8), 10 + b)
             points[f"decode_b{b}"] = round(v, 1)
 
     line = {
-        "metric": f"decode tok/s, Qwen3-{args.shape} shape, batch {args.batch}, {T}-token prompts",
+        "metric": f"decode tok/s, Qwen3-{args.shape} shape, batch {batch}, {T}-token prompts",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dname, "data": "synthetic: random token ids, random weights N(0, 0.02^2), norms 1 + N(0, 0.1^2)",
-        "config": {
-            "model": f"Qwen3-{args.shape} shape", "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers,
-            "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
-            "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-            "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps, "tied_head": cfg.tie_word_embeddings,
-            "global_batch": args.batch, "prompt_len": T, "seq_len": args.context, "kv_block": args.block_size,
-            "parallelism": "single GPU", "graphs": not args.eager,
-        },
+        "config": config_of(args, cfg, full_layers, global_batch=batch, prompt_len=T, seq_len=context),
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
         "points": points,
+        "step_ms": {"p50": round(percentile(step_ms, 0.5), 4), "p95": round(percentile(step_ms, 0.95), 4)},
     }
+    if peaks:
+        line["measured"] = dict(peaks, roofline_frac=round(achieved / peaks["hbm_read_GBs"], 4),
+                                prefill_frac=round(pre_flops / pre_s / (peaks["gemm_bf16_TFLOPs"] * 1e12), 4))
+    line["gemm_choices"] = llm.gemm_choices()
+    if args.gemm_choices:
+        import os
+        if not os.path.isfile(args.gemm_choices):
+            llm.save_gemm_choices(args.gemm_choices)
     print(json.dumps(line), flush=True)
     return 0
+
+
+def bench_workload(args):
+    """The serving workloads: every request queued at once, prompts in portions beside decoding requests."""
+    import torch
+    from nanohybrid_vlm_amd import SamplingParams
+
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    dname = "bf16" if args.dtype == "bfloat16" else "fp32"
+    if args.shape != "32b":
+        batch, n_out = args.batch or 32, args.output_tokens or 128
+        longest = args.prompt_tokens or 4096
+        g = torch.Generator().manual_seed(14)
+        lengths = torch.randint(128, longest + 1, (batch,), generator=g).tolist()
+        context = args.context or (longest + n_out)
+        pages = sum(-(-(n + n_out) // args.block_size) for n in lengths) + 1
+        cache = {"num_kvcache_blocks": pages}
+        workload = f"{batch} requests, prompts uniform in [128, {longest}], {n_out} new tokens each, portions of 2048"
+    else:
+        batch, n_out = args.batch or 16, args.output_tokens or 256
+        longest = args.prompt_tokens or 8192
+        lengths = [longest] * batch
+        context = args.context or (longest + n_out)
+        cache = {"num_kvcache_blocks": -1}            # the cache takes what is left of the device's memory
+        workload = f"{batch} requests of {longest} prompt tokens, {n_out} new tokens each, cache sized from free memory"
+    llm, cfg, full_layers = build_llm(args, batch, max_num_batched_tokens=2048, max_model_len=context, **cache)
+    weight_bytes, kv_per_token, matrix_flops = model_bytes_and_flops(cfg, itemsize)
+    peaks = measured_peaks(args)
+    sp = SamplingParams(temperature=0.0, max_tokens=n_out, ignore_eos=True)
+
+    def once(seed):
+        prompts = [random_prompts(1, n, cfg.vocab_size, seed + i)[0] for i, n in enumerate(lengths)]
+        for p in prompts:
+            llm.add_request(p, sp)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        steps = []
+        while not llm.is_finished():
+            _, st = llm.step()
+            steps.append(st)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, steps
+
+    once(1000)                                        # untimed: graphs are recorded, products measured
+    wall, steps = once(2000)
+    decode_only = [s for s in steps if s.num_prefill_tokens == 0]
+    with_prompts = [s for s in steps if s.num_prefill_tokens > 0]
+    generated = batch * n_out
+    decode_s = sum(s.seconds for s in decode_only)
+    decode_tokens = sum(s.num_decode_tokens for s in decode_only)
+    live_tokens = sum(lengths) + generated / 2.0      # the cache that a decode-only step reads, about
+    decode_ms = decode_s / max(len(decode_only), 1) * 1e3
+    achieved = (weight_bytes + live_tokens * kv_per_token) / (decode_ms * 1e-3) / 1e9 if decode_only else 0.0
+    prompt_s = sum(s.seconds for s in with_prompts)
+    prompt_tokens = sum(s.num_prefill_tokens + s.num_decode_tokens for s in with_prompts)
+    stats = llm.get_memory_stats()
+    line = {
+        "metric": f"generated tok/s, Qwen3-{args.shape} shape, {workload}",
+        "value": round(generated / wall, 1), "unit": "tok/s", "n_gpus": 1, "steps": len(steps), "warmup": len(steps),
+        "ms_per_step": round(wall / len(steps) * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dname, "data": "synthetic: random token ids, random weights N(0, 0.02^2), norms 1 + N(0, 0.1^2)",
+        "config": config_of(args, cfg, full_layers, global_batch=batch, prompt_len=longest, seq_len=context,
+                            token_budget=2048, cache_pages=stats["groups"][0]["pages"]),
+        "prefill": {"value": round(prompt_tokens / prompt_s, 1) if prompt_s else None, "tokens": sum(lengths),
+                    "ms": round(prompt_s * 1e3, 3), "frac": round(matrix_flops * prompt_tokens / prompt_s / PEAK_FLOPS[dname], 4) if prompt_s else None},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": {"decode_only_tok_s": round(decode_tokens / decode_s, 1) if decode_s else None,
+                   "decode_only_ms_per_step": round(decode_ms, 4), "wall_s": round(wall, 3),
+                   "preemptions": llm.scheduler.num_preemptions},
+        "step_ms": {"p50": round(percentile([s.seconds * 1e3 for s in steps], 0.5), 4),
+                    "p95": round(percentile([s.seconds * 1e3 for s in steps], 0.95), 4)},
+    }
+    if peaks:
+        line["measured"] = dict(peaks, roofline_frac=round(achieved / peaks["hbm_read_GBs"], 4))
+    line["gemm_choices"] = llm.gemm_choices()
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
+        return 2
+    serving = args.workload == "serving" or (args.workload == "auto" and args.shape in ("14b", "32b"))
+    if serving:
+        return bench_workload(args)
+    return bench_decode_points(args)
 
 
 if __name__ == "__main__":

@@ -60,6 +60,11 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
                     help="requests with a common start share the full pages that hold it")
     ap.add_argument("--plugin", action="append", metavar="MODULE",
                     help="a module to import first: it may register architectures and parts of its own; repeatable")
+    ap.add_argument("--gemm-choices", metavar="FILE",
+                    help="how each shape of matrix product is done: read from FILE if it exists (nothing is timed then), "
+                         "written to it at the end otherwise")
+    ap.add_argument("--no-measure-gemms", action="store_true",
+                    help="time no matrix product: shapes follow --gemm-choices, else the fixed rule")
 
 
 def _import_plugins(names) -> None:
@@ -98,7 +103,13 @@ def _make_llm(args):
                kvcache_block_size=args.block_size, num_kvcache_blocks=args.num_blocks, max_num_seqs=args.max_num_seqs,
                max_model_len=args.max_model_len, scheduler_policy=args.scheduler_policy, seed=args.seed,
                enable_prefix_cache=args.enable_prefix_cache, max_graph_batch=args.max_graph_batch,
-               run_ahead=not args.no_run_ahead)
+               run_ahead=not args.no_run_ahead, gemm_choices=args.gemm_choices, measure_gemms=not args.no_measure_gemms)
+
+
+def _save_choices(llm, args) -> None:
+    import os
+    if args.gemm_choices and not os.path.isfile(args.gemm_choices):
+        llm.save_gemm_choices(args.gemm_choices)
 
 
 def _percentile(values, q):
@@ -123,6 +134,7 @@ def cmd_generate(args) -> int:
         return 2
     sp = SamplingParams(temperature=args.temperature, max_tokens=args.output_tokens, ignore_eos=args.ignore_eos)
     outputs = llm.generate(prompts, sp, use_tqdm=not args.quiet)
+    _save_choices(llm, args)
     result = [{"prompt": p, **o} for p, o in zip(prompts, outputs)]
     text = json.dumps(result, indent=2)
     if args.output:
@@ -188,6 +200,7 @@ def cmd_bench(args) -> int:
         timer.__exit__(None, None, None)
         print(times.table())
     print(json.dumps({"memory": llm.get_memory_stats()}), flush=True)
+    _save_choices(llm, args)
     if args.output:
         Path(args.output).write_text(json.dumps({"model": args.model, "mode": args.mode, "dtype": args.dtype,
                                                  "token_budget": args.token_budget, "results": results}, indent=2))

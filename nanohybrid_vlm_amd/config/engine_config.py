@@ -30,6 +30,10 @@ class EngineConfig:
     num_kvcache_blocks: int = -1                # -1: sized from free memory
     num_state_slots: int = -1                   # -1: max_num_seqs
     enable_prefix_cache: bool = False           # requests with a common start share its full pages
+    # bfloat16 matrix products are done the fastest way measured (own kernel or one of the library's algorithms), timed
+    # once per shape and process; which way wins can differ from start to start, and with it the last bits of the logits.
+    measure_gemms: bool = True                  # False: nothing is timed; shapes follow gemm_choices, else the fixed rule
+    gemm_choices: str | None = None             # a JSON file of choices: read if it exists (and then nothing is timed), see LLM.save_gemm_choices
     dtype: str = "bfloat16"                     # "bfloat16" or "float32" (true 32-bit everywhere)
     seed: int = 0                               # default seed of temperature sampling
     device: str = "cuda:0"                      # the one GPU

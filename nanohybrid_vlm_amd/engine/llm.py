@@ -119,6 +119,7 @@ class LLM:
         if built_model is None and not os.path.isdir(model):
             raise FileNotFoundError(f"model folder '{model}' does not exist")
         arch, typed, built = built_model if built_model is not None else (None, None, None)
+        self._set_up_gemm_choices(cfg)
         self.runner = ModelRunner(
             model, dtype=cfg.dtype, device=cfg.device, page_size=cfg.kvcache_block_size,
             num_pages=None if cfg.num_kvcache_blocks == -1 else cfg.num_kvcache_blocks,
@@ -142,6 +143,41 @@ class LLM:
         self._completed_metrics: list[RequestMetrics] = []
         self._ahead = None               # a decoding step issued before its tokens were known to the host (see step)
         self.num_steps_ahead = 0         # steps that were already under way when their turn came
+
+    # ------------------------------------------------------------------ how matrix products are done
+    @staticmethod
+    def _set_up_gemm_choices(cfg: EngineConfig) -> None:
+        """Tells the kernel library whether it may time matrix products, and gives it a table of choices made by an
+        earlier run. With a table (or with measuring off) the same kernels run in every process: logits are the same
+        bit for bit from start to start, and no step pays for a measurement."""
+        import json
+        from ..native import ops
+        backend = ops.backend()
+        if not hasattr(backend, "load_choices"):
+            return                                     # (a stand-in for the kernels has nothing to choose)
+        backend.measuring_allowed = bool(cfg.measure_gemms)
+        if cfg.gemm_choices and os.path.isfile(cfg.gemm_choices):
+            with open(cfg.gemm_choices) as f:
+                backend.load_choices(json.load(f))
+            backend.measuring_allowed = False
+
+    def gemm_choices(self) -> dict:
+        """How each shape of matrix product met so far is done ("M,N,K,float result,gated" -> -1 own kernel, -2 the
+        rule, or a library algorithm's number)."""
+        from ..native import ops
+        backend = ops.backend()
+        return backend.choices_table() if hasattr(backend, "choices_table") else {}
+
+    def save_gemm_choices(self, path: str | None = None) -> str:
+        """Writes the choices made so far to ``path`` (default: the engine option ``gemm_choices``); a later run
+        started with ``gemm_choices=path`` does every product the same way and times nothing."""
+        import json
+        path = path or self.config.gemm_choices
+        if not path:
+            raise ValueError("no file named: pass a path or start the engine with gemm_choices=PATH")
+        with open(path, "w") as f:
+            json.dump(self.gemm_choices(), f, indent=1, sort_keys=True)
+        return path
 
     # ------------------------------------------------------------------ requests
     def add_request(self, prompt, sampling_params: SamplingParams | None = None) -> int:
@@ -270,7 +306,9 @@ class LLM:
         return result
 
     def get_memory_stats(self) -> dict:
-        return self.runner.get_memory_stats()
+        stats = self.runner.get_memory_stats()
+        stats["gemm_choices"] = self.gemm_choices()
+        return stats
 
     def get_completed_request_metrics(self) -> list[RequestMetrics]:
         out, self._completed_metrics = self._completed_metrics, []

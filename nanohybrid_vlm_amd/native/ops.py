@@ -19,7 +19,7 @@ import torch
 from . import library
 
 CORE_SOURCES = ["error.hip", "elementwise.hip", "gemm_generic.hip", "gemm_skinny_bf16.hip", "gemm_fewrows_bf16.hip", "attention_generic.hip",
-                "sampling.hip"]
+                "sampling.hip", "measure.hip"]
 BLAS_SOURCES = ["error.hip", "gemm_library.hip"]                                                   # the vendor's matrix library, algorithm by number
 BLAS_LINK = ["-lhipblaslt"]
 ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip", "attention_prefill_bf16.hip"]      # compiled once per head size
@@ -105,6 +105,7 @@ class NativeBackend:
     planned_context = 0           # > 0 while a HIP graph is recorded: the lengths to plan for (the batch's own are bounds)
     measure_linears = False       # True: a product of few rows and a shape not seen before is timed in every way there is (see _choose)
     measure_many_rows = True      # a product of more than library_rows rows is timed in the third step that meets its shape
+    measuring_allowed = True      # False: nothing is ever timed; a shape follows the table that was loaded, or the rule
     step_number = 0               # counted by the engine, one per eager step
 
     def __init__(self):
@@ -275,7 +276,7 @@ class NativeBackend:
         float_result = out.dtype == torch.float32
         key = (M, N, K, float_result, gated)
         known = self.chosen.get(key)
-        if known is not None or torch.cuda.is_current_stream_capturing():
+        if known is not None or not self.measuring_allowed or torch.cuda.is_current_stream_capturing():
             return known
         many = M > self.library_rows
         if many:
@@ -365,6 +366,24 @@ class NativeBackend:
                   f"of {len(runs)} ways); taken: {name.get(how, how)}", file=sys.stderr, flush=True)
         return how
 
+    # -- the table of choices, so that a process can run by what another one measured --
+    def choices_table(self) -> dict[str, int]:
+        """What has been chosen so far, by shape: "M,N,K,float result,gated" -> -1 (own kernel), -2 (the rule:
+        ``torch.mm``) or the number of a library algorithm."""
+        return {",".join(str(int(v)) for v in key): how for key, how in sorted(self.chosen.items())}
+
+    def load_choices(self, table: dict[str, int]) -> None:
+        """Takes a table as ``choices_table`` gives it. An entry that names a library algorithm is checked against
+        the library's list for the shape when it is first used (``nhv_library_gemm`` refuses a number beyond it)."""
+        for text, how in table.items():
+            parts = text.split(",")
+            if len(parts) != 5:
+                raise KernelError(f"a product's shape is 'M,N,K,float result,gated', got '{text}'")
+            M, N, K, f, g = (int(v) for v in parts)
+            if not isinstance(how, int) or how < RULE:
+                raise KernelError(f"choice {how!r} for the product '{text}' is neither -1, -2 nor an algorithm's number")
+            self.chosen[(M, N, K, bool(f), bool(g))] = how
+
     def end_measurements(self) -> None:
         """Gives the scratch memory of the measurements back (what was measured stays known)."""
         self._sweep = None
@@ -420,6 +439,33 @@ class NativeBackend:
         piece_index = torch.empty((n, pieces), dtype=torch.int32, device=logits.device)
         self._call("nhv_sample", _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(tokens), n, V, _ptr(piece_value),
                    _ptr(piece_index), _stream())
+
+
+def measured_peaks(device="cuda:0", read_bytes: int = 4 << 30, gemm_size: int = 8192) -> dict:
+    """What this very GPU gives, for fractions beside those of the published peaks: the rate of a kernel that only
+    reads ``read_bytes`` from memory (each byte once, far more than the caches hold), and the rate of a bfloat16
+    matrix product of ``gemm_size``^3 by the vendor's library. The shortest of five runs each."""
+    b = backend()
+    data = torch.empty(read_bytes // 1024 * 1024, dtype=torch.uint8, device=device).zero_()
+    sink = torch.zeros(1, dtype=torch.float32, device=device)
+
+    def shortest(run, n=5):
+        best = float("inf")
+        for _ in range(n + 1):                      # (the first run is a warm-up)
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            run()
+            end.record()
+            end.synchronize()
+            best = min(best, start.elapsed_time(end) * 1e-3)
+        return best
+
+    read_s = shortest(lambda: b._call("nhv_measure_read", _ptr(data), _ptr(sink), ctypes.c_size_t(data.numel()), _stream()))
+    del data
+    a = torch.randn(gemm_size, gemm_size, dtype=torch.bfloat16, device=device)
+    c = torch.empty_like(a)
+    gemm_s = shortest(lambda: torch.mm(a, a.t(), out=c))
+    return {"hbm_read_GBs": read_bytes // 1024 * 1024 / read_s / 1e9, "gemm_bf16_TFLOPs": 2.0 * gemm_size ** 3 / gemm_s / 1e12}
 
 
 class KernelTimes:

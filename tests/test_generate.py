@@ -317,3 +317,56 @@ def test_a_configuration_with_random_weights_in_place_of_a_folder(emulated_kerne
         LLM("some folder", random_weights=1, **options)
     with pytest.raises(ValueError, match="dtype"):
         LLM(dict(TINY_B), random_weights=1, device="cpu", dtype="float16")
+
+
+@pytest.mark.gpu
+def test_pinned_gemm_choices_make_bfloat16_runs_repeat_bit_for_bit(model_folders, tmp_path):
+    """Which kernel does a bfloat16 matrix product (own, or one of the library's algorithms) is normally decided by
+    a timing, once per shape and process. With ``measure_gemms=False`` nothing is timed and every shape follows the
+    fixed rule; with ``gemm_choices=FILE`` a run does every product the way an earlier run chose. Either way two
+    engines give the same logits bit for bit."""
+    import json
+    from nanohybrid_vlm_amd.engine.runner import StepEntry
+    from nanohybrid_vlm_amd.native import ops
+    folder = model_folders["D"]
+    cfg, _ = plain.read_model_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, 700 + n) for n in (40, 3, 100, 17, 9, 64, 30, 5, 12, 21)]
+    options = dict(dtype="bfloat16", kvcache_block_size=64, num_kvcache_blocks=64, max_num_batched_tokens=256, max_model_len=256)
+
+    def logits_of(llm):
+        """Prompt portions of many rows, then single tokens of ten requests through a recorded step."""
+        runner = llm.runner
+        first = runner.step([StepEntry(("probe", i), p, [len(p) - 1]) for i, p in enumerate(prompts)])
+        second = runner.step([StepEntry(("probe", i), [7 + i], [0]) for i in range(len(prompts))])
+        third = runner.step([StepEntry(("probe", i), [9 + i], [0]) for i in range(len(prompts))])
+        for i in range(len(prompts)):
+            runner.finish(("probe", i))
+        return torch.cat([first, second, third]).cpu()
+
+    backend = ops.backend()
+    # nothing measured: the rule, twice
+    runs = []
+    for _ in range(2):
+        backend.chosen.clear()
+        llm = LLM(folder, measure_gemms=False, **options)
+        runs.append(logits_of(llm))
+        assert llm.gemm_choices() == {} and backend.chosen == {}
+    assert torch.equal(runs[0], runs[1])
+    # measured once, written down, followed by the next engine
+    path = str(tmp_path / "choices.json")
+    backend.chosen.clear()
+    llm = LLM(folder, gemm_choices=path, **options)
+    measured = logits_of(llm)
+    table = llm.gemm_choices()
+    assert table and all(len(k.split(",")) == 5 for k in table), "the recorded step's shapes were measured"
+    assert llm.get_memory_stats()["gemm_choices"] == table
+    llm.save_gemm_choices()
+    assert json.load(open(path)) == table
+    backend.chosen.clear()
+    llm = LLM(folder, gemm_choices=path, **options)
+    assert backend.measuring_allowed is False and llm.gemm_choices() == table
+    again = logits_of(llm)
+    assert llm.gemm_choices() == table, "nothing was measured in the second run"
+    assert torch.equal(again, measured)
+    backend.measuring_allowed = True
+    backend.chosen.clear()
