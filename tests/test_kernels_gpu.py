@@ -354,6 +354,44 @@ def test_prefill_attention_bfloat16(ops, Hq, Hkv, D, page, window):
     torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("window", [None, 5000])
+def test_attention_over_32768_keys(ops, window):
+    """Both bfloat16 attention kernels at 32,768 keys on pages of 256 (128 pages a request, hundreds of splits to
+    merge, block tables past what a block keeps in LDS at smaller pages), against the float64 computation: a single
+    token at the end of 32,768 keys beside one after 9,001; and portions of 130 and 64 tokens that end at 32,768
+    and 20,000 keys. In every request one early key is made to stand out for one head's queries, so that a key lost
+    far from the end shows."""
+    Hq, Hkv, D, page = 8, 2, 128, 256
+    scale = D ** -0.5
+    for lens, q_lens in ([[32768, 9001], [1, 1]], [[32768, 20000], [130, 64]]):
+        q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=41, scale=1.0)
+        # key 777 (and key n - 4100, inside a window of 5,000) of every request points where head 3's queries point
+        g = torch.Generator().manual_seed(5)
+        direction = torch.randn(D, generator=g)
+        direction = (direction / direction.norm()).to(torch.bfloat16)
+        row = 0
+        for r, (n, nq) in enumerate(zip(lens, q_lens)):
+            for far in (777, n - 4100):
+                ks[r][far, 0] = ks[r][far, 0] + 14.0 * direction          # head 3 reads key/value head 0
+                pid = int(bt[r, far // page])
+                kc[pid, far % page, 0] = ks[r][far, 0].cuda()
+            qs[r][:, 3] = qs[r][:, 3] + 14.0 * direction
+            q[row:row + nq, 3] = qs[r][:, 3].cuda()
+            row += nq
+        out = ops.paged_attention(q, kc, vc, batch, bt, scale, window)
+        ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, window)
+        torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
+        # (the input does what it is meant to: nearly all of the softmax's weight of head 3's last query lies on the
+        # keys that stand out, so an output that agrees with the reference has found them)
+        for r, n in enumerate(lens):
+            scores = (ks[r][:, 0].double() @ qs[r][-1, 3].double()) * scale
+            if window:
+                scores[:n - window] = float("-inf")
+            weight = torch.softmax(scores, 0)
+            far = [n - 4100] if window else [777, n - 4100]
+            assert weight[far].sum() > 0.95
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("page", [8, 64, 256])
 def test_attention_finds_one_far_key(ops, dtype, page):
