@@ -187,3 +187,80 @@ def test_noise_of_the_extreme_bit_patterns():
         below = sum(1 for b in range(n - 1, n - 200, -1) if plain.noise_of_bits(b) < x) if x < 1e-5 else None
         if below is not None:
             assert abs(below / n - (1 - math.exp(-x))) <= 1.0 / n
+
+
+# ---------------------------------------------------------------- readings that no library routine fixes
+def _variant_logits(cfg, w, toks, first_position=0, norm_after_rotation=False, post_norm=False, scale_power=-0.5):
+    """The model from the plain part functions with three switches, each a plausible misreading of the reference:
+    the per-head norms of q and k after the rotation instead of before it (nanovllm/models/qwen3.py:82-85), a
+    post-norm block instead of the pre-norm one with the addition carried on (qwen3.py:152-159), and another power
+    of the head size as the scale (qwen3.py:39). With all switches off it is the plain implementation."""
+    Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    eps, theta = cfg["rms_norm_eps"], cfg["rope_theta"]
+    T = len(toks)
+    pos = torch.arange(first_position, first_position + T)
+    r = w["model.embed_tokens.weight"][toks]
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+
+        def attention(x):
+            q = (x @ w[p + "self_attn.q_proj.weight"].T).view(T, Hq, D)
+            k = (x @ w[p + "self_attn.k_proj.weight"].T).view(T, Hkv, D)
+            v = (x @ w[p + "self_attn.v_proj.weight"].T).view(T, Hkv, D)
+            qn, kn = w[p + "self_attn.q_norm.weight"], w[p + "self_attn.k_norm.weight"]
+            if norm_after_rotation:
+                q = plain.rms_norm(plain.apply_rope(q, pos, theta), qn, eps)
+                k = plain.rms_norm(plain.apply_rope(k, pos, theta), kn, eps)
+            else:
+                q = plain.apply_rope(plain.rms_norm(q, qn, eps), pos, theta)
+                k = plain.apply_rope(plain.rms_norm(k, kn, eps), pos, theta)
+            return plain.causal_attention(q, k, v, D ** scale_power).reshape(T, Hq * D) @ w[p + "self_attn.o_proj.weight"].T
+
+        def feed_forward(x):
+            return plain.swiglu(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+
+        if post_norm:
+            r = plain.rms_norm(r + attention(r), w[p + "input_layernorm.weight"], eps)
+            r = plain.rms_norm(r + feed_forward(r), w[p + "post_attention_layernorm.weight"], eps)
+        else:
+            r = r + attention(plain.rms_norm(r, w[p + "input_layernorm.weight"], eps))
+            r = r + feed_forward(plain.rms_norm(r, w[p + "post_attention_layernorm.weight"], eps))
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
+    return plain.rms_norm(r, w["model.norm.weight"], eps) @ head.T
+
+
+@pytest.mark.parametrize("cfg,seed", [(TINY_A, 0), (TINY_B, 1)])
+def test_each_pin_rejects_the_misreading_it_is_there_for(cfg, seed):
+    w = _random_weights(cfg, seed)
+    toks = torch.randint(0, cfg["vocab_size"], (19,), generator=torch.Generator().manual_seed(seed)).tolist()
+    # the function with its switches off is the plain implementation
+    torch.testing.assert_close(_variant_logits(cfg, w, toks), plain.logits(cfg, w, toks), rtol=1e-5, atol=1e-6)
+
+    # 1. q/k norm before the rotation. The norm's weight differs from entry to entry, so a norm *after* the rotation
+    # mixes the turned pairs with unequal weights and the scores depend on where the sequence starts: the pin
+    # "only distances between positions count" holds for the right order and fails for the wrong one.
+    def shift_error(**switches):
+        return (_variant_logits(cfg, w, toks, first_position=0, **switches)
+                - _variant_logits(cfg, w, toks, first_position=37, **switches)).abs().max().item()
+    assert shift_error() < 2e-5
+    assert shift_error(norm_after_rotation=True) > 50 * 2e-5
+
+    # 2. the pre-norm block with the addition carried to the next norm: with every layer's output projections at
+    # zero the residual stream stays the embedding and the logits are norm(embedding) . head^T. A post-norm block
+    # norms the stream itself in every layer and gives other logits.
+    dead = {n: (torch.zeros_like(t) if n.endswith(("o_proj.weight", "down_proj.weight")) else t) for n, t in w.items()}
+    e = w["model.embed_tokens.weight"]
+    head = e if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
+    ref = F.rms_norm(e[toks], (cfg["hidden_size"],), w["model.norm.weight"], cfg["rms_norm_eps"]) @ head.T
+    torch.testing.assert_close(_variant_logits(cfg, dead, toks), ref, rtol=1e-5, atol=1e-6)
+    assert (_variant_logits(cfg, dead, toks, post_norm=True) - ref).abs().max() > 1e-2
+
+    # 3. the scale is head_dim ** -0.5, which is the library routine's own default: attention of whole heads without
+    # rotation equals F.scaled_dot_product_attention called *without* a scale; another power of the head size does not
+    D = cfg["head_dim"]
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(11, 3, D, generator=g) for _ in range(3))
+    lib = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True).transpose(0, 1)
+    torch.testing.assert_close(plain.causal_attention(q, k, v, D ** -0.5), lib, rtol=1e-5, atol=1e-6)
+    assert (plain.causal_attention(q, k, v, D ** -1.0) - lib).abs().max() > 1e-2
+    assert (_variant_logits(cfg, w, toks, scale_power=-1.0) - plain.logits(cfg, w, toks)).abs().max() > 1e-4
