@@ -42,8 +42,31 @@
 // the loads into LDS and the barrier of each tile. More waves do not help either: one row tile a wave, tiles of
 // 32 keys and four waves per SIMD (128 registers, 36 KB of LDS a block) reached 550 TFLOP/s, since every wave then
 // reads all keys and values from LDS for half as many rows.
+//
+// Where the time goes (counters of one run of 8,192 new tokens, 32 query and 8 key/value heads of 128): the matrix
+// cores are busy 36 % of the time; a wave issues 198 other vector instructions for every 64 matrix instructions of a
+// tile (332 before the mask became a compile-time choice and the rescaling a real branch: that change alone took the
+// kernel from 806 to 943 TFLOP/s at 8,192 tokens and from 441 to 537 at 2,048, bit for bit the same results), 67
+// scalar ones and 49 reads of LDS. With the loads of all tiles but the first left out (wrong results, timing only) the
+// kernel takes 16 % less time, without the barriers as well 20 % less: four fifths of the time is the tiles'
+// arithmetic itself, in which the matrix instructions of one wave and the vector instructions of the other on the
+// same SIMD overlap only in part (a microbenchmark: 8 matrix and 24 multiply-add instructions interleaved in one
+// wave take 222 clocks where they take 153 and 148 apart). Measured and not kept after that: the rows' sums of P
+// taken by the matrix cores (a V^T operand of ones; 32 additions fewer and 4 matrix instructions more a tile): 2 %;
+// the tiles' loads as buffer loads whose address is a scalar descriptor and a 32-bit offset (no 64-bit vector
+// additions): nothing; two groups of four waves a block that take the block's key tiles in turn and add up through
+// LDS at the end, so that a block's chain of tiles is half as long (one block of eight waves a compute unit): 3 to
+// 15 % more time at every length, since both groups then wait for their loads at the same moments, which two
+// independent blocks on a compute unit do not; blocks of eight waves with one row tile each, four buffers of tiles
+// and loads three tiles ahead, one block a compute unit: the same 2,048-token time and 15 to 25 % more at 3,072
+// tokens and beyond (every wave reads every tile's keys and values from LDS whatever its number of rows: 256 KB
+// a tile for eight waves, which is what such a block's tile then takes); the reads from LDS written one operand
+// ahead of the products that use them, with and without the order pinned by scheduler group barriers: nothing.
+// (When kernels are compared, the first one or two of a process run up to a tenth slower than later ones: what is
+// compared has to be run in turn, more than once.)
 #include "nhv_common.h"
 #include <math.h>
+#include <type_traits>
 
 #ifndef NHV_HEAD_DIM
 #error "compile with -DNHV_HEAD_DIM=<head size>"
@@ -237,7 +260,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     }
   };
 
-  auto compute = [&](int kb, const bf16_t* k_s, const bf16_t* v_s) {
+  // MASKED (a type, so that each call site names a compile-time choice): whether some key of the tile is hidden from
+  // some row of the wave. Tiles wholly inside every row's range, which are nearly all, run code without the
+  // comparisons: as a run-time flag the test cost three to four instructions for every score in every tile.
+  auto compute = [&](auto masked, int kb, const bf16_t* k_s, const bf16_t* v_s) {
+    constexpr bool MASKED = decltype(masked)::value;
     // ---- scores of the tile's keys for this wave's rows: every K operand serves all row tiles
     floatx4 s4[RT][KT];
 #pragma unroll
@@ -253,8 +280,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
         for (int r = 0; r < RT; ++r) s4[r][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[r][s], s4[r][kt], 0, 0, 0);
       }
     }
-    // tiles wholly inside every row's range need no mask
-    const bool need_mask = kb + BN - 1 > wave_lo_pos || kb < wave_max_lo;
     bf16x8 pa[RT][KT / 2];                                 // P of keys (32 a + 4 grp + j) and (32 a + 16 + 4 grp + j)
     float alpha[RT];
     bool grow[RT];
@@ -267,7 +292,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          if (need_mask) {
+          if (MASKED) {
             const int key = kb + kt * 16 + grp * 4 + j;
             if (key > row_pos[r] || key < row_lo[r]) s4[r][kt][j] = -INFINITY;
           }
@@ -297,17 +322,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
       l_part[r] = l_part[r] * alpha[r] + psum;
       m_run[r] = m_new;
     }
+    // The outputs are rescaled only when a reference has moved: a branch of the whole wave, taken rarely. (Written
+    // as a condition inside the loop over the output tiles, the compiler made a multiply and a select of it for
+    // every output entry in every tile, 128 instructions a tile; the empty statement keeps the branch a branch.)
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+      if (grow[r]) {
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o[r][dt][j] *= alpha[r];
+      }
     // this lane points at key 4 grp + col / 4 of a 16-key sub-tile, entries 4 (col % 4).. of the 16-entry block dt
     const int tr_key = grp * 4 + (col >> 2);
     const int tr_piece = (col & 3) >> 1, tr_half = (col & 1) * 4;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
-#pragma unroll
-      for (int r = 0; r < RT; ++r)
-        if (grow[r]) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) o[r][dt][j] *= alpha[r];
-        }
 #pragma unroll
       for (int a = 0; a < KT / 2; ++a) {
         // this lane's eight summation slots: keys 32 a + 4 grp + (0..3) and 32 a + 16 + 4 grp + (0..3), entry dt * 16 + col
@@ -325,6 +356,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     }
   };
 
+  auto run = [&](int kb, const bf16_t* k_s, const bf16_t* v_s) {
+    if (kb + BN - 1 > wave_lo_pos || kb < wave_max_lo) compute(std::true_type{}, kb, k_s, v_s);
+    else compute(std::false_type{}, kb, k_s, v_s);
+  };
+
   // tiles alternate between the two buffers; the loop is written out for both so that every load and read names
   // its buffer (the compiler then knows that the loads under way do not touch the tile being read)
   const int kb0 = (key_lo / BN) * BN;
@@ -333,12 +369,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                                       // this tile has arrived, the other buffer has been read
     if (kb + BN <= key_hi) issue(kb + BN, k_s1, v_s1);
-    if (live && kb <= wave_hi) compute(kb, k_s0, v_s0);    // a whole-wave decision; the wave still meets the barriers
+    if (live && kb <= wave_hi) run(kb, k_s0, v_s0);        // a whole-wave decision; the wave still meets the barriers
     if (kb + BN > key_hi) break;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (kb + 2 * BN <= key_hi) issue(kb + 2 * BN, k_s0, v_s0);
-    if (live && kb + BN <= wave_hi) compute(kb + BN, k_s1, v_s1);
+    if (live && kb + BN <= wave_hi) run(kb + BN, k_s1, v_s1);
   }
   if (!live) return;
 #pragma unroll
