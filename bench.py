@@ -15,6 +15,9 @@ decoding at batch 1 and 64; ``step_ms`` the timed steps' median and 95th percent
 once, prompts fed in portions of 2,048 tokens beside the decoding requests (continuous batching).
 ``--shape 32b``: 16 requests of 8,192 prompt tokens and 256 generated tokens, the cache sized from free memory.
 For these two ``value`` is generated tokens a second over the whole run, prompts included; a step is an engine step.
+
+``--workload projections`` is a diagnosis, not the benchmark: a layer's matrix products alone, cold, beside a kernel
+that only reads the same bytes (see ``bench_projections``).
 """
 import argparse
 import json
@@ -25,15 +28,20 @@ PEAK_HBM_GBS = 8000.0            # MI355X, published
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}   # dense MFMA, published
 
 
+def _int_or_list(text):
+    return int(text) if text.isdigit() else text      # (a list of row counts, "1,8,64", for --workload projections)
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=192)
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--batch", type=int, default=None, help="requests decoding side by side (8b: 8, 14b: 32, 32b: 16)")
+    ap.add_argument("--batch", type=_int_or_list, default=None, help="requests decoding side by side (8b: 8, 14b: 32, 32b: 16)")
     ap.add_argument("--shape", default="8b")
-    ap.add_argument("--workload", default="auto", choices=("auto", "points", "serving"),
-                    help="points: decode at a fixed batch after equal prompts (8b by default); serving: the 14b / 32b workloads")
+    ap.add_argument("--workload", default="auto", choices=("auto", "points", "serving", "projections"),
+                    help="points: decode at a fixed batch after equal prompts (8b by default); serving: the 14b / 32b workloads; "
+                         "projections: a layer's matrix products alone against a kernel that only reads the same bytes")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (same layer sizes)")
     ap.add_argument("--prompt-tokens", type=int, default=None, help="8b: 2048; 32b: 8192; 14b: the longest prompt, 4096")
     ap.add_argument("--output-tokens", type=int, default=None, help="14b: 128; 32b: 256")
@@ -44,6 +52,8 @@ def parse_args():
     ap.add_argument("--no-measured-peaks", action="store_true", help="skip the measurement of what this GPU gives")
     ap.add_argument("--eager", action="store_true", help="no HIP graphs")
     ap.add_argument("--max-graph-batch", type=int, default=None, help="largest decode batch that replays a graph")
+    ap.add_argument("--residual-dtype", default="float32", choices=("float32", "model"),
+                    help="the residual stream between layers: float32, or rounded to the element type as the reference does")
     ap.add_argument("--gemm-choices", default=None, help="JSON file of matrix-product choices to follow (and to write if absent)")
     return ap.parse_args()
 
@@ -64,7 +74,7 @@ def build_llm(args, max_seqs, **options):
     if args.layers:
         raw["num_hidden_layers"] = args.layers
     llm = LLM(raw, random_weights=0, dtype=args.dtype, kvcache_block_size=args.block_size, max_num_seqs=max_seqs,
-              enforce_eager=args.eager, gemm_choices=args.gemm_choices,
+              enforce_eager=args.eager, gemm_choices=args.gemm_choices, residual_dtype=args.residual_dtype,
               **({"max_graph_batch": args.max_graph_batch} if args.max_graph_batch else {}), **options)
     return llm, llm.runner.cfg, full_layers
 
@@ -300,12 +310,100 @@ def bench_workload(args):
     return 0
 
 
+def bench_projections(args):
+    """How near a decode step's matrix products are to what the memory gives them: for each of a layer's four weight
+    matrices and the head, a chain of products with different weights of that size (1 GB or more in all, so that no
+    weight is found in a cache), recorded into a graph as in a decode step, done as the engine does them (the own
+    kernel or the library algorithm that the engine's measurement picks) and by the own kernels alone, beside a chain
+    of a kernel that only reads the same bytes. Rows: 1, 8 and 64 (``--batch`` for another list, e.g. 1,16)."""
+    import ctypes
+    import torch
+    from nanohybrid_vlm_amd.config.registry import named_shapes, resolve_architecture
+    from nanohybrid_vlm_amd.native import ops
+
+    raw = dict(named_shapes()[args.shape])
+    cfg = resolve_architecture(raw).parse_config(raw)
+    H, I, D = cfg.hidden_size, cfg.intermediate_size, cfg.head_dim
+    shapes = [("qkv", (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * D, H, False), ("o", H, cfg.num_attention_heads * D, False),
+              ("gate_up", 2 * I, H, True), ("down", H, I, False), ("head", cfg.vocab_size, H, False)]
+    rows = [int(m) for m in str(args.batch).split(",")] if args.batch else [1, 8, 64]
+    b = ops.backend()
+    stream = torch.cuda.Stream()
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    table = {}
+
+    def chain_us(run, count):
+        """Microseconds a call, of ``count`` calls recorded into one graph; the shortest of five replays."""
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            run()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                run()
+            graph.replay()
+            torch.cuda.synchronize()
+            best = float("inf")
+            for _ in range(5):
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                graph.replay()
+                end.record()
+                end.synchronize()
+                best = min(best, start.elapsed_time(end))
+        return best * 1e3 / count
+
+    print(f"{'product':8s} {'MB':>7s} {'rows':>4s} {'engine us':>10s} {'TB/s':>5s} {'own us':>8s} {'TB/s':>5s} {'read us':>8s} {'TB/s':>5s}  engine/read",
+          flush=True)
+    for name, N, K, gated in shapes:
+        nbytes = N * K * 2
+        count = min(32, max(4, -(-(1 << 30) // nbytes)))
+        weights = [torch.randn(N, K, device="cuda", dtype=torch.bfloat16) * 0.02 for _ in range(count)]
+
+        def read():
+            for w in weights:
+                b._call("nhv_measure_read", ctypes.c_void_p(w.data_ptr()), ctypes.c_void_p(sink.data_ptr()),
+                        ctypes.c_size_t(nbytes // 1024 * 1024), ops._stream())
+        read_us = chain_us(read, count)
+        for M in rows:
+            x = torch.randn(M, K, device="cuda", dtype=torch.bfloat16)
+            float_result = name == "head"
+
+            def products():
+                for w in weights:
+                    if gated:
+                        ops.gated_linear(x, w)
+                    else:
+                        ops.linear(x, w, out_dtype=torch.float32 if float_result else None)
+            b.measure_linears, b.own_kernels_only = True, False
+            products()                                 # (the first call of a shape measures it; the answer is kept)
+            b.measure_linears = False
+            b.end_measurements()
+            engine_us = chain_us(products, count)
+            b.own_kernels_only = True
+            own_us = chain_us(products, count)
+            b.own_kernels_only = False
+            table[f"{name}_m{M}"] = {"engine_us": round(engine_us, 2), "own_us": round(own_us, 2), "read_us": round(read_us, 2)}
+            print(f"{name:8s} {nbytes / 1e6:7.1f} {M:4d} {engine_us:10.1f} {nbytes / engine_us / 1e6:5.2f} {own_us:8.1f} "
+                  f"{nbytes / own_us / 1e6:5.2f} {read_us:8.1f} {nbytes / read_us / 1e6:5.2f}  {engine_us / read_us:.2f}", flush=True)
+        del weights
+    for M in rows:
+        layer = [table[f"{n}_m{M}"] for n in ("qkv", "o", "gate_up", "down")]
+        print(f"a layer's four products at {M} rows: engine {sum(t['engine_us'] for t in layer):.1f} us, own kernels "
+              f"{sum(t['own_us'] for t in layer):.1f} us, reading alone {sum(t['read_us'] for t in layer):.1f} us", flush=True)
+    print(json.dumps({"metric": f"a layer's matrix products against reads of the same bytes, Qwen3-{args.shape} shape",
+                      "unit": "us", "dtype": "bf16", "table": table, "gemm_choices": b.choices_table()}), flush=True)
+    return 0
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
         return 2
     serving = args.workload == "serving" or (args.workload == "auto" and args.shape in ("14b", "32b"))
+    if args.workload == "projections":
+        return bench_projections(args)
     if serving:
         return bench_workload(args)
     return bench_decode_points(args)

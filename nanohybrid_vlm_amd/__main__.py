@@ -63,6 +63,9 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--gemm-choices", metavar="FILE",
                     help="how each shape of matrix product is done: read from FILE if it exists (nothing is timed then), "
                          "written to it at the end otherwise")
+    ap.add_argument("--residual-dtype", choices=("float32", "model"), default="float32",
+                    help="the residual stream between layers: kept in float32, or rounded to the model's element type "
+                         "after every addition as the reference does")
     ap.add_argument("--no-measure-gemms", action="store_true",
                     help="time no matrix product: shapes follow --gemm-choices, else the fixed rule")
 
@@ -103,7 +106,8 @@ def _make_llm(args):
                kvcache_block_size=args.block_size, num_kvcache_blocks=args.num_blocks, max_num_seqs=args.max_num_seqs,
                max_model_len=args.max_model_len, scheduler_policy=args.scheduler_policy, seed=args.seed,
                enable_prefix_cache=args.enable_prefix_cache, max_graph_batch=args.max_graph_batch,
-               run_ahead=not args.no_run_ahead, gemm_choices=args.gemm_choices, measure_gemms=not args.no_measure_gemms)
+               run_ahead=not args.no_run_ahead, gemm_choices=args.gemm_choices, measure_gemms=not args.no_measure_gemms,
+               residual_dtype=args.residual_dtype)
 
 
 def _save_choices(llm, args) -> None:

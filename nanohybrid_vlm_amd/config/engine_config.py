@@ -35,6 +35,9 @@ class EngineConfig:
     measure_gemms: bool = True                  # False: nothing is timed; shapes follow gemm_choices, else the fixed rule
     gemm_choices: str | None = None             # a JSON file of choices: read if it exists (and then nothing is timed), see LLM.save_gemm_choices
     dtype: str = "bfloat16"                     # "bfloat16" or "float32" (true 32-bit everywhere)
+    # the residual stream between layers in a bfloat16 run: "float32" keeps the unrounded sum; "model" rounds it to
+    # bfloat16 after every addition, as the reference does (and reads and writes a third fewer bytes in every norm)
+    residual_dtype: str = "float32"
     seed: int = 0                               # default seed of temperature sampling
     device: str = "cuda:0"                      # the one GPU
 
@@ -42,6 +45,8 @@ class EngineConfig:
         if self.dtype not in _DTYPES:
             raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {self.dtype!r}")
         self.dtype = _DTYPES[self.dtype]
+        if self.residual_dtype not in ("float32", "model"):
+            raise ValueError("residual_dtype must be 'float32' or 'model'")
         if self.scheduler_policy not in ("decode_first", "prefill_first"):
             raise ValueError("scheduler_policy must be 'decode_first' or 'prefill_first'")
         if self.max_prefill_wait_ms < 0:

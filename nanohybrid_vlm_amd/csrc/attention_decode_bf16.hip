@@ -202,14 +202,19 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
     m_run = m_new;
     __syncthreads();                                   // the tile is written
     // ---- O^T += V^T P^T
+    // (the outputs are rescaled only when the reference has moved: a branch of the whole wave; written as a condition
+    // inside the loop over the output tiles it became a multiply and a select for every output entry in every round)
+    if (grow) {
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
+    }
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
       const int drow = dt * 16 + col;
       const int swz = ((drow >> 3) & SWZ_MASK) << 2;
-      if (grow) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
-      }
 #pragma unroll
       for (int a = 0; a < KT / 2; ++a) {
         const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vt_s + drow * VPITCH + ((a * 32 + grp * 4) ^ swz));

@@ -48,7 +48,7 @@ class ModelRunner:
                  num_pages: int | None = None, num_state_slots: int = 512, gpu_memory_utilization: float = 0.9,
                  max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None, use_graphs: bool = False,
                  max_model_len: int | None = None, max_graph_batch: int = 64, poison_freed_pages: bool = False,
-                 share_prefixes: bool = False):
+                 share_prefixes: bool = False, residual_float32: bool = True):
         """``model``/``arch``/``cfg`` may be given ready-made (weights already bound)
         instead of being read from ``model_dir``."""
         if dtype not in _TORCH_DTYPES:
@@ -63,6 +63,10 @@ class ModelRunner:
             load_weights(model, arch, cfg, model_dir, self.dtype, self.device)
         self.arch, self.cfg, self.model = arch, cfg, model
         self.model.to(self.device)
+        # an engine option that parts carry as an attribute: whether the residual stream keeps float32 between layers
+        for part in self.model.walk():
+            if hasattr(part, "residual_float32"):
+                part.residual_float32 = bool(residual_float32)
         # what the engine above needs to know of the model comes from the model's description, not from the
         # architecture's typed configuration (whose fields are the architecture's own affair)
         self.vocab_size = model.spec.vocab_size

@@ -543,10 +543,12 @@ def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, residual: torch.Tensor | None = None,
-            start_residual: bool = False):
+            start_residual: bool = False, residual_float32: bool = True):
     """``rmsnorm(x, w, eps)``: the norm of x.
-    ``residual=r``: r += x in place (in float) and the norm of the sum is returned.
-    ``start_residual=True``: returns (norm of x, a new float32 residual holding x)."""
+    ``residual=r``: r += x in place (the sum is taken in float and normed unrounded; r keeps it in its own element
+    type) and the norm of the sum is returned.
+    ``start_residual=True``: returns (norm of x, the residual that later norms add to): a new float32 tensor holding
+    x, or, with ``residual_float32=False``, x itself (which later calls then add to in place)."""
     _need(x.dim() == 2, "rmsnorm: x must be [tokens, width]")
     _dense(x, "rmsnorm: x")
     _dense(w, "rmsnorm: weight", (x.shape[1],))
@@ -556,6 +558,9 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, residual: torch.Tensor
     y = torch.empty_like(x)
     if start_residual:
         _need(residual is None, "rmsnorm: a residual is either started or added to")
+        if not residual_float32 and x.dtype != torch.float32:
+            backend().rmsnorm(x, None, 0, w, y, float(eps))
+            return y, x
         residual = torch.empty(x.shape, dtype=torch.float32, device=x.device)
         backend().rmsnorm(x, residual, 2, w, y, float(eps))
         return y, residual

@@ -74,6 +74,12 @@ class Part:
             setattr(self, name.replace(".", "_"), tensor)
 
     # -- walking the tree -------------------------------------------------
+    def walk(self):
+        """This part and every part below it."""
+        yield self
+        for child in self.children().values():
+            yield from child.walk()
+
     def all_param_specs(self, prefix: str = "") -> dict[str, ParamSpec]:
         out = {prefix + k: v for k, v in self.param_specs().items()}
         for cname, child in self.children().items():

@@ -12,6 +12,12 @@ class RMSNorm(Part):
     """y = x / sqrt(mean(x^2) + eps) * weight; with a residual the sum is normed
     and carried on (layernorm.py:28-40)."""
 
+    # True: the residual stream is carried in float32 whatever the rows' element type, so the sum goes from layer
+    # to layer unrounded. False: it is carried in the rows' element type, rounded after every addition, as the
+    # reference carries it (layernorm.py:34-40; the norm itself still takes the unrounded float sum). An engine
+    # option, set on every norm of a model by the runner.
+    residual_float32 = True
+
     def __init__(self, size: int, eps: float):
         self.size = size
         self.eps = eps
@@ -24,10 +30,8 @@ class RMSNorm(Part):
         return ops.rmsnorm(x, self.weight, self.eps)
 
     def forward_start(self, x: torch.Tensor):
-        """The first norm of a model: returns (norm(x), x as the residual that later norms add to).
-        The residual is kept in float32 whatever the rows' element type, so the sum is
-        carried from layer to layer without rounding."""
-        return ops.rmsnorm(x, self.weight, self.eps, start_residual=True)
+        """The first norm of a model: returns (norm(x), x as the residual that later norms add to)."""
+        return ops.rmsnorm(x, self.weight, self.eps, start_residual=True, residual_float32=self.residual_float32)
 
     def forward_add(self, x: torch.Tensor, residual: torch.Tensor):
         """Returns (norm(x + residual), x + residual); ``residual`` is updated in place."""

@@ -76,6 +76,13 @@ def test_rmsnorm_float32_residual_with_bfloat16_rows(ops):
     assert torch.equal(res, s)
     ref = s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + 1e-6) * w.float()
     torch.testing.assert_close(y2.float(), ref, **tol(torch.bfloat16))
+    # the residual in the rows' own type: it starts as x itself, and a sum is rounded when it is stored
+    y3, res3 = ops.rmsnorm(x, w, 1e-6, start_residual=True, residual_float32=False)
+    assert res3 is x and torch.equal(y3, y)
+    before = x.clone()
+    y4 = ops.rmsnorm(x2, w, 1e-6, residual=res3)
+    assert torch.equal(res3, (before.float() + x2.float()).bfloat16())
+    torch.testing.assert_close(y4.float(), ref, **tol(torch.bfloat16))
 
 
 def test_rmsnorm_float32_weight_with_bfloat16_rows(ops):

@@ -355,3 +355,39 @@ def test_pool_of_a_replay():
             assert pages_for(counted, page) >= sum(-(-n // page) for n in lengths), (page, lengths)
 
 
+
+
+def _replay_with_rounded_residual(folder, device, graphs):
+    """The residual stream carried in bfloat16, rounded after every addition as the reference carries it
+    (nanovllm/layers/layernorm.py:34-40), instead of in float32: the same four ways against the plain implementation."""
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    cfg, _ = plain.read_model_folder(folder)
+    requests = _requests(cfg["vocab_size"])
+    want = _plain_logits(folder, requests)
+    tol = tolerance_for("bfloat16", want)
+    results = {}
+    for mode, steps in [("whole", rc.whole(requests)), ("tail", rc.tail_decoded(requests)),
+                        ("portions", rc.portions(requests)), ("mixed", rc.mixed(requests))]:
+        pages = rc.peak_tokens(steps, 8) // 8
+        runner = _poisoned(ModelRunner(folder, dtype="bfloat16", device=device, page_size=8, num_pages=pages, num_state_slots=4,
+                                       use_graphs=graphs, max_model_len=160, poison_freed_pages=True, residual_float32=False))
+        assert all(not part.residual_float32 for part in runner.model.walk() if hasattr(part, "residual_float32"))
+        results[mode] = rc.run_in_process(runner, steps)
+        _check(results[mode], want, tol, f"rounded residual, {mode}")
+    return results
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_rounded_residual_on_emulated_kernels(model_folders, emulated_kernels, name):
+    _replay_with_rounded_residual(model_folders[name], "cpu", graphs=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_rounded_residual_on_gpu(model_folders, name, graphs):
+    results = _replay_with_rounded_residual(model_folders[name], "cuda:0", graphs)
+    for mode in ("tail", "portions", "mixed"):
+        for rid in results["whole"]:
+            d = max_abs_diff(results[mode][rid], results["whole"][rid])
+            assert d <= 0.5 * TOLERANCE["bfloat16"], f"rounded residual, {mode} against whole: request {rid}: {d:.3e}"
