@@ -62,6 +62,19 @@
 // tokens and beyond (every wave reads every tile's keys and values from LDS whatever its number of rows: 256 KB
 // a tile for eight waves, which is what such a block's tile then takes); the reads from LDS written one operand
 // ahead of the products that use them, with and without the order pinned by scheduler group barriers: nothing.
+// Two further attempts, both giving the same bits as this kernel and neither kept. The exponentials of a 16-key
+// sub-tile taken against the references as they stand, right behind its matrix instructions and issued in turn with
+// those of the next sub-tile (the order pinned by scheduler group barriers; a tile in which a row grows is done again
+// the plain way): 8 to 10 % more time at every length, with the order pinned or left to the compiler. And blocks of
+// eight waves, two row tiles each, one block a compute unit, with three buffers of tiles and the loads two tiles
+// ahead (issued by inline assembly: the compiler, which counts the loads into each LDS array itself, otherwise waits
+// for all of them before the first read of a tile): the same time where all blocks have long key ranges (2,048 tokens
+// after 26,000: 882 against 888 us) and 4 to 25 % more for portions without earlier keys, whose one block a unit cannot
+// pair a long key range with a short one. So the kernel waits neither for its tiles to arrive nor for a better order
+// of its own instructions: its time is about that of its matrix instructions plus that of its vector instructions,
+// one after the other (per 64-key tile and wave 64 x 16 clocks and about 1,200, measured 2,550 for the two waves of a
+// SIMD together), as if the two kinds did not overlap; a microbenchmark of both kinds interleaved in one wave shows
+// half of the vector instructions' time hidden at best.
 // (When kernels are compared, the first one or two of a process run up to a tenth slower than later ones: what is
 // compared has to be run in turn, more than once.)
 #include "nhv_common.h"
