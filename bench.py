@@ -404,6 +404,9 @@ def main():
     serving = args.workload == "serving" or (args.workload == "auto" and args.shape in ("14b", "32b"))
     if args.workload == "projections":
         return bench_projections(args)
+    if isinstance(args.batch, str):
+        print(f"bench.py: --batch {args.batch}: a list of row counts goes with --workload projections only", flush=True)
+        return 2
     if serving:
         return bench_workload(args)
     return bench_decode_points(args)
