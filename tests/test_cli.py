@@ -63,3 +63,41 @@ def test_bench_refuses_more_than_one_gpu():
                           cwd=REPO, capture_output=True, text=True, timeout=300)
     assert proc.returncode == 2
     assert len(proc.stdout.strip().splitlines()) == 1 and "one GPU" in proc.stdout
+
+
+def _bench(*args, timeout=600):
+    proc = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), *args], cwd=REPO, capture_output=True, text=True,
+                          timeout=timeout)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = [line for line in proc.stdout.splitlines() if line.startswith("{")]
+    assert len(lines) == 1, proc.stdout[-2000:]
+    return json.loads(lines[0]), proc.stdout
+
+
+@pytest.mark.gpu
+def test_bench_program_on_a_tiny_shape():
+    """The measurement program's three kinds of run, on a tiny shape: the line's fields are there and add up."""
+    line, _ = _bench("--shape", "tinyB", "--steps", "6", "--warmup", "2", "--batch", "3", "--prompt-tokens", "40",
+                     "--context", "64", "--block-size", "16")
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "prefill", "roofline", "points", "step_ms", "measured"):
+        assert key in line, key
+    assert line["n_gpus"] == 1 and line["steps"] == 6 and line["dtype"] == "bf16" and line["value"] > 0
+    assert abs(line["value"] - 3 / (line["ms_per_step"] * 1e-3)) <= 0.01 * line["value"]
+    config = line["config"]
+    assert len(config) <= 20 and all(not isinstance(v, (dict, list)) for v in config.values())
+    assert config["hidden"] == 96 and config["layers"] == config["layers_of_shape"] == 3 and config["vocab"] == 389
+    assert set(line["prefill"]) == {"value", "tokens", "ms", "frac"} and line["prefill"]["tokens"] == 40
+    roofline = line["roofline"]
+    assert roofline["bound"] == "hbm" and roofline["peak"] == 8000.0
+    assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-3
+    assert set(line["points"]) == {"decode_b1", "decode_b64"} and all(v > 0 for v in line["points"].values())
+    # a serving workload: every request queued at once, prompts in portions beside decoding requests
+    line, _ = _bench("--shape", "tinyB", "--workload", "serving", "--batch", "5", "--prompt-tokens", "150",
+                     "--output-tokens", "8", "--block-size", "16", "--no-measured-peaks")
+    assert line["value"] > 0 and line["points"]["decode_only_tok_s"] > 0 and len(line["config"]) <= 20
+    # the diagnosis of a layer's products
+    line, text = _bench("--shape", "tinyB", "--workload", "projections", "--batch", "1,5")
+    assert set(line["table"]) == {f"{name}_m{m}" for name in ("qkv", "o", "gate_up", "down", "head") for m in (1, 5)}
+    assert all(v["engine_us"] > 0 and v["read_us"] > 0 for v in line["table"].values())
+    assert "a layer's four products at 5 rows" in text
