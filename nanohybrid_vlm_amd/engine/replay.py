@@ -10,6 +10,16 @@ A step is a dict, one line of JSON in a trace file:
 are wanted; all entries of a step are one batch. ``end``: requests that are over
 after this step; what they hold in the cache is given back.
 
+A whole trace may also come as one JSON object that names the requests' tokens once and
+then says, step by step, how many of its next tokens each request feeds:
+
+    {"requests": {"a": [5, 17, 3, 9], "b": [1, 2]}, "steps": [[{"req": "a", "n": 3}], [{"req": "a", "n": 1}, {"req": "b", "n": 2}]],
+     "dtype": "float32", "block_size": 64, "num_blocks": 8, "model": "DIR"}        (or "shape": "tinyB", "seed": 1)
+
+``steps_of_trace`` turns it into steps of the first kind: the logits of every fed position are
+wanted, and a request ends with its last token. ``bin/trace_run --trace FILE --out X.safetensors``
+then writes ``{request: [its length, vocab]}``.
+
 ``bin/trace_run`` and the tests' in-process replays both go through ``replay_step``,
 so the program and the tests drive the engine in the same way. The reference has
 nothing like it; the nearest is stepping its engine by hand
@@ -69,3 +79,45 @@ def replay(runner: ModelRunner, steps) -> dict:
                 row += n
         runner.cache.check()
     return {rid: torch.cat(p) for rid, p in parts.items()}
+
+
+def steps_of_trace(trace: dict) -> list[dict]:
+    """The steps of a trace that is one object (see the module's text), as the records that ``replay_step`` takes.
+    Everything that is wrong with the trace is an error here, before any step has run."""
+    requests = trace.get("requests")
+    if not isinstance(requests, dict) or not requests or not isinstance(trace.get("steps"), list):
+        raise ValueError("a trace holds 'requests': {id: [token ids]} and 'steps': [[{'req': id, 'n': count}, ...], ...]")
+    fed = {rid: 0 for rid in requests}
+    records = []
+    for number, step in enumerate(trace["steps"]):
+        entries, ended = [], []
+        for item in step:
+            rid, n = item.get("req"), item.get("n")
+            if rid not in requests:
+                raise ValueError(f"step {number}: request {rid!r} is not among the trace's requests")
+            if not isinstance(n, int) or n <= 0 or fed[rid] + n > len(requests[rid]):
+                raise ValueError(f"step {number}: request {rid!r} cannot feed {n!r} tokens after {fed[rid]} of its "
+                                 f"{len(requests[rid])}")
+            entries.append({"id": rid, "tokens": list(requests[rid][fed[rid]:fed[rid] + n]), "want": list(range(n))})
+            fed[rid] += n
+            if fed[rid] == len(requests[rid]):
+                ended.append(rid)
+        records.append({"step": number, "entries": entries, "end": ended})
+    unfinished = sorted(str(rid) for rid, n in fed.items() if n != len(requests[rid]))
+    if unfinished:
+        raise ValueError(f"the steps do not feed all tokens of request(s) {', '.join(unfinished)}")
+    return records
+
+
+def peak_tokens_of(records: list[dict], unit: int = 64) -> int:
+    """The most tokens that live requests hold at any time in these steps, each request's count rounded up to a
+    multiple of ``unit``: what ``make_runner`` sizes the cache for."""
+    held: dict = {}
+    peak = 0
+    for record in records:
+        for e in record.get("entries") or []:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        peak = max(peak, sum(-(-n // unit) * unit for n in held.values()))
+        for rid in record.get("end") or []:
+            held.pop(rid, None)
+    return peak

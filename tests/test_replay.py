@@ -391,3 +391,67 @@ def test_rounded_residual_on_gpu(model_folders, name, graphs):
         for rid in results["whole"]:
             d = max_abs_diff(results[mode][rid], results["whole"][rid])
             assert d <= 0.5 * TOLERANCE["bfloat16"], f"rounded residual, {mode} against whole: request {rid}: {d:.3e}"
+
+
+# ---------------------------------------------------------------- a whole trace as one object
+
+def _as_whole_trace(requests, steps, **more):
+    """The steps of ``replay_cases`` in the other form: the requests' tokens once, and per step how many each feeds."""
+    return dict({"requests": requests, "steps": [[{"req": e["id"], "n": len(e["tokens"])} for e in st["entries"]]
+                                                 for st in steps]}, **more)
+
+
+def test_steps_of_a_whole_trace():
+    from nanohybrid_vlm_amd.engine.replay import peak_tokens_of, steps_of_trace
+    requests = {"a": [5, 17, 3, 9], "b": [1, 2]}
+    records = steps_of_trace({"requests": requests, "steps": [[{"req": "a", "n": 3}], [{"req": "a", "n": 1}, {"req": "b", "n": 2}]]})
+    assert records == [{"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 1, 2]}], "end": []},
+                       {"step": 1, "entries": [{"id": "a", "tokens": [9], "want": [0]},
+                                               {"id": "b", "tokens": [1, 2], "want": [0, 1]}], "end": ["a", "b"]}]
+    assert peak_tokens_of(records) == 128 and peak_tokens_of(records, unit=2) == 6
+    mixed = rc.mixed(_requests(50))
+    assert steps_of_trace(_as_whole_trace(_requests(50), mixed)) == [
+        dict(st, entries=[dict(e, want=list(range(len(e["tokens"])))) for e in st["entries"]]) for st in mixed]
+    assert peak_tokens_of(mixed, 8) == rc.peak_tokens(mixed, 8)
+    for bad, what in [({"requests": requests, "steps": [[{"req": "c", "n": 1}]]}, "not among"),
+                      ({"requests": requests, "steps": [[{"req": "a", "n": 5}]]}, "cannot feed"),
+                      ({"requests": requests, "steps": [[{"req": "a", "n": 0}]]}, "cannot feed"),
+                      ({"requests": requests, "steps": [[{"req": "a", "n": 4}]]}, "do not feed all tokens of request(s) b"),
+                      ({"requests": {}, "steps": []}, "a trace holds")]:
+        with pytest.raises(ValueError, match=what.replace("(", r"\(").replace(")", r"\)")):
+            steps_of_trace(bad)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program_with_a_whole_trace(model_folders, dtype, tmp_path):
+    """``bin/trace_run --trace trace.json --out logits.safetensors``: the trace names model, element type, page size
+    and pages itself; the file holds every request's logits at all its positions."""
+    from safetensors.torch import load_file
+    folder = model_folders["B"]
+    cfg, _ = plain.read_model_folder(folder)
+    requests = _requests(cfg["vocab_size"])
+    want = _plain_logits(folder, requests)
+    steps = rc.mixed(requests)
+    trace = _as_whole_trace(requests, steps, model=folder, dtype=dtype, block_size=16,
+                            num_blocks=rc.peak_tokens(steps, 16) // 16)
+    path = str(tmp_path / "trace.json")
+    with open(path, "w") as f:
+        json.dump(trace, f)
+    out = str(tmp_path / "logits.safetensors")
+    proc = subprocess.run([sys.executable, os.path.join(REPO, "bin", "trace_run"), "--trace", path, "--out", out],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(steps))]
+    got = load_file(out)
+    assert set(got) == set(requests) and all(got[rid].dtype == torch.float32 for rid in got)
+    _check(got, want, tolerance_for(dtype, want), f"whole trace, {dtype}")
+    # a random model named by shape and seed, files a step: the same steps as lines give the same files
+    trace = _as_whole_trace(requests, steps, shape="tinyB", seed=5, dtype="float32", block_size=16)
+    with open(path, "w") as f:
+        json.dump(trace, f)
+    out_dir = str(tmp_path / "files")
+    proc = subprocess.run([sys.executable, os.path.join(REPO, "bin", "trace_run"), "--trace", path, "--out", out_dir],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert sorted(os.listdir(out_dir), key=lambda n: int(n.split(".")[0])) == [f"{i}.f32" for i in range(len(steps))]
