@@ -35,7 +35,7 @@ def _int_or_list(text):
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=192)
+    ap.add_argument("--steps", type=int, default=240)     # with the 16 warm-up steps: 256 generated tokens a request
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=_int_or_list, default=None, help="requests decoding side by side (8b: 8, 14b: 32, 32b: 16)")
     ap.add_argument("--shape", default="8b")
