@@ -619,3 +619,80 @@ def test_library_products_refuse_what_they_cannot_do(ops):
                       ctypes.byref(ctypes.c_int()), lib=backend.blas_lib())
     backend._library_product(x, w, out, 0)
     torch.testing.assert_close(out.double(), x.double() @ w.double().T, **tol(torch.bfloat16))
+
+
+# ---------------------------------------------------------------- sizes drawn at random (seeded)
+# The kernels choose waves, loads in flight, tiles a block and split lengths from the sizes by rules; these cases walk
+# over the rules' borders at sizes nobody picked by hand.
+
+def _random_product_sizes(seed, count, max_rows):
+    import random
+    rnd_ = random.Random(seed)
+    sizes = []
+    while len(sizes) < count:
+        M = rnd_.randint(1, max_rows)
+        N = rnd_.choice([rnd_.randint(1, 600), rnd_.randint(600, 9000), rnd_.randint(9000, 40000)])
+        K = 8 * rnd_.choice([rnd_.randint(1, 64), rnd_.randint(64, 1000), rnd_.randint(1000, 3300)])
+        if N * K <= 48_000_000:
+            sizes.append((M, N, K))
+    return sizes
+
+
+@pytest.mark.parametrize("M,N,K", _random_product_sizes(1, 40, 16) + _random_product_sizes(2, 12, 64))
+def test_products_of_few_rows_at_random_sizes(ops, M, N, K):
+    x = rnd(M, K, dtype=torch.bfloat16, seed=44)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=45, scale=K ** -0.5)
+    ref = x.double() @ w.double().T
+    backend = ops.backend()
+    backend.own_kernels_only = True                          # the own kernels, whatever a measurement would choose
+    try:
+        got = ops.linear(x, w, out_dtype=torch.float32)
+        torch.testing.assert_close(got.double(), ref, rtol=1e-4, atol=2e-4)
+        assert torch.equal(got, ops.linear(x, w, out_dtype=torch.float32))
+        torch.testing.assert_close(ops.linear(x, w).double(), ref, **tol(torch.bfloat16))
+        if N % 2 == 0:
+            g, u = ref[:, :N // 2], ref[:, N // 2:]
+            torch.testing.assert_close(ops.gated_linear(x, w).double(), g * torch.sigmoid(g) * u, **tol(torch.bfloat16))
+    finally:
+        backend.own_kernels_only = False
+
+
+def _random_attention_cases(seed, count):
+    import random
+    rnd_ = random.Random(seed)
+    cases = []
+    for _ in range(count):
+        Hkv = rnd_.choice([1, 2, 3, 8])
+        G = rnd_.choice([1, 2, 3, 4, 5, 8, 16])
+        D = 16 * rnd_.randint(1, 8) if rnd_.random() < 0.8 else 256
+        page = rnd_.choice([3, 8, 16, 48, 64, 256])
+        window = rnd_.choice([None, None, rnd_.randint(1, 40), rnd_.randint(41, 900)])
+        cases.append((Hkv * G, Hkv, D, page, window, rnd_.randint(0, 10 ** 6)))
+    return cases
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,page,window,seed", _random_attention_cases(3, 16))
+def test_attention_kernels_at_random_sizes(ops, Hq, Hkv, D, page, window, seed):
+    """Both bfloat16 attention kernels (single tokens; portions beside single tokens) at head counts, group sizes,
+    head sizes, page sizes, windows and lengths drawn at random."""
+    import random
+    rnd_ = random.Random(seed)
+    scale = D ** -0.5
+    # single tokens: the split-key kernel
+    lens = [rnd_.choice([rnd_.randint(1, 70), rnd_.randint(70, 700), rnd_.randint(700, 2600)]) for _ in range(rnd_.randint(1, 9))]
+    q_lens = [1] * len(lens)
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=seed, scale=1.5)
+    out = ops.paged_attention(q, kc, vc, batch, bt, scale, window)
+    torch.testing.assert_close(out.double().cpu(), _attention_reference(qs, ks, vs, lens, q_lens, scale, window),
+                               **tol(torch.bfloat16))
+    # portions with and without earlier keys beside single tokens: the matrix-core kernel for prompts
+    lens = [rnd_.randint(1, 1200) for _ in range(rnd_.randint(1, 5))]
+    q_lens = [rnd_.choice([1, n, rnd_.randint(1, n)]) for n in lens]
+    q_lens[0] = max(2, min(lens[0], q_lens[0])) if lens[0] > 1 else 1
+    if max(q_lens) == 1:
+        lens.append(300)
+        q_lens.append(77)
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=seed + 1, scale=1.5)
+    out = ops.paged_attention(q, kc, vc, batch, bt, scale, window)
+    torch.testing.assert_close(out.double().cpu(), _attention_reference(qs, ks, vs, lens, q_lens, scale, window),
+                               **tol(torch.bfloat16))
