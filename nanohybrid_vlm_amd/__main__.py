@@ -51,6 +51,8 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--num-blocks", type=int, default=-1, help="pages of the cache (-1: from free memory)")
     ap.add_argument("--max-num-seqs", type=int, default=512)
     ap.add_argument("--max-graph-batch", type=int, default=64, help="decode steps of up to this many requests replay a graph")
+    ap.add_argument("--max-graph-tokens", type=int, default=256,
+                    help="other steps (prompt portions, alone or beside decoded tokens) of up to this many tokens replay a graph; 0: none")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="every step is issued only when the tokens of the step before are known to the host")
     ap.add_argument("--max-model-len", type=int, default=4096)
@@ -105,7 +107,7 @@ def _make_llm(args):
                max_num_batched_tokens=args.token_budget, gpu_memory_utilization=args.gpu_memory_utilization,
                kvcache_block_size=args.block_size, num_kvcache_blocks=args.num_blocks, max_num_seqs=args.max_num_seqs,
                max_model_len=args.max_model_len, scheduler_policy=args.scheduler_policy, seed=args.seed,
-               enable_prefix_cache=args.enable_prefix_cache, max_graph_batch=args.max_graph_batch,
+               enable_prefix_cache=args.enable_prefix_cache, max_graph_batch=args.max_graph_batch, max_graph_tokens=args.max_graph_tokens,
                run_ahead=not args.no_run_ahead, gemm_choices=args.gemm_choices, measure_gemms=not args.no_measure_gemms,
                residual_dtype=args.residual_dtype)
 

@@ -24,6 +24,7 @@ class EngineConfig:
     gpu_memory_utilization: float = 0.9
     enforce_eager: bool = False                 # True: no HIP graphs for decode
     max_graph_batch: int = 64                   # decode steps of up to this many requests replay a graph
+    max_graph_tokens: int = 256                 # so do other steps (prompt portions, alone or beside decoded tokens) of up to this many tokens; 0: none
     run_ahead: bool = True                      # a decode step that is bound to follow is issued before the host knows the tokens it feeds
     eos: int = -1                               # filled from config.json when -1
     kvcache_block_size: int = 256               # tokens in a page (any positive number)
@@ -67,6 +68,8 @@ class EngineConfig:
             raise ValueError("num_state_slots must be -1 or positive")
         if self.max_graph_batch <= 0:
             raise ValueError("max_graph_batch must be positive")
+        if self.max_graph_tokens < 0:
+            raise ValueError("max_graph_tokens must not be negative")
 
     @classmethod
     def field_names(cls) -> set[str]:

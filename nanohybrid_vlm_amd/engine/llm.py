@@ -126,7 +126,7 @@ class LLM:
             num_state_slots=cfg.max_num_seqs if cfg.num_state_slots == -1 else cfg.num_state_slots,
             gpu_memory_utilization=cfg.gpu_memory_utilization, max_num_batched_tokens=cfg.max_num_batched_tokens,
             model=built, arch=arch, cfg=typed, use_graphs=not cfg.enforce_eager, max_model_len=cfg.max_model_len,
-            share_prefixes=cfg.enable_prefix_cache, max_graph_batch=cfg.max_graph_batch,
+            share_prefixes=cfg.enable_prefix_cache, max_graph_batch=cfg.max_graph_batch, max_graph_tokens=cfg.max_graph_tokens,
             residual_float32=cfg.residual_dtype == "float32")
         cfg.num_kvcache_blocks = self.runner.num_pages
         # max_model_len is capped by the model's positions (nanovllm/config.py:420-423); both, and the token that

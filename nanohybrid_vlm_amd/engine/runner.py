@@ -48,7 +48,7 @@ class ModelRunner:
                  num_pages: int | None = None, num_state_slots: int = 512, gpu_memory_utilization: float = 0.9,
                  max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None, use_graphs: bool = False,
                  max_model_len: int | None = None, max_graph_batch: int = 64, poison_freed_pages: bool = False,
-                 share_prefixes: bool = False, residual_float32: bool = True):
+                 share_prefixes: bool = False, residual_float32: bool = True, max_graph_tokens: int = 256):
         """``model``/``arch``/``cfg`` may be given ready-made (weights already bound)
         instead of being read from ``model_dir``."""
         if dtype not in _TORCH_DTYPES:
@@ -78,7 +78,7 @@ class ModelRunner:
                              "poison_freed_pages would destroy it")
         self.share_prefixes = share_prefixes
         self._make_cache(page_size, num_pages, num_state_slots, gpu_memory_utilization, max_num_batched_tokens,
-                         graph_rows=max_graph_batch if use_graphs else 0)
+                         graph_rows=max_graph_batch if use_graphs else 0, graph_tokens=max_graph_tokens if use_graphs else 0)
         self._pinned = None
         self._pinned_free = None
         # a debugging aid: pages that are given back are filled with NaN, so that a read of a page that a
@@ -97,11 +97,21 @@ class ModelRunner:
         # batch sizes that have a graph: a step is padded to the next one
         self.graph_buckets = self._bucket_sizes(max_graph_batch)
         self._graphs: dict[int, dict | None] = {}     # None: the bucket's graph failed its check
+        # Short steps of any make (portions of prompts, beside decoded tokens or alone) are bound by their launches as
+        # well: some 350 kernels of a few microseconds each against 15 to 20 us of host work a launch. A step of up to
+        # ``max_graph_tokens`` tokens in which every request wants at most one place replays a graph too, recorded for
+        # (tokens, requests) rounded up to the next sizes of ``mixed_token_buckets`` and the decode buckets: the tokens
+        # that fill the bucket belong to a request of their own, whose keys are the zeros of the spare page and which
+        # stores nothing, and the requests that fill it have no tokens. 0 switches this off.
+        self.max_graph_tokens = max_graph_tokens if self.use_graphs else 0
+        self.mixed_token_buckets = self._token_bucket_sizes(self.max_graph_tokens)
+        self.mixed_request_buckets = [b for b in (1, 4, 16) if b < max_graph_batch] + [max_graph_batch]
+        self._mixed_graphs: dict[tuple[int, int], dict | None] = {}
         self.graph_check = torch.equal                # (replay, eager) -> bool; a test replaces it to force a refusal
         self.graphs_rerecorded = 0                    # graphs recorded again because the contexts had outgrown their layout
 
     # ------------------------------------------------------------------ cache
-    def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens, graph_rows=0):
+    def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens, graph_rows=0, graph_tokens=0):
         needs = self.model.cache_needs()
         windows: list[int | None] = []                 # one group per distinct window
         entry_group: dict[int, int] = {}
@@ -132,7 +142,7 @@ class ModelRunner:
         page_bytes = sum(2 * page_size * n.num_kv_heads * n.head_dim * item
                          for n in needs if isinstance(n, PagedKVNeed))
         if num_pages is None:
-            num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens, graph_rows)
+            num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens, graph_rows, graph_tokens)
         self.num_pages = num_pages
         groups = [PagedGroupSpec(name="all keys" if w is None else f"window {w}", page_size=page_size,
                                  num_pages=num_pages, window=w) for w in windows]
@@ -157,7 +167,7 @@ class ModelRunner:
                 views[i] = CacheView(kind="none")
         self.model.attach_cache(views)
 
-    def _pages_from_free_memory(self, page_bytes, utilization, max_tokens, graph_rows) -> int:
+    def _pages_from_free_memory(self, page_bytes, utilization, max_tokens, graph_rows, graph_tokens=0) -> int:
         """budget = total * utilization - used - room for a step's activations - room for the recorded steps
         (nanovllm/engine/model_runner.py:654-699,839-861; the reference measures the room with a warm-up pass,
         here it is computed from the layer sizes). The weights and the state pools are allocated already and
@@ -175,12 +185,22 @@ class ModelRunner:
         # every recorded batch size keeps its own logits and a step's activations of that many rows
         buckets = [b for b in self._bucket_sizes(graph_rows)] if graph_rows else []
         recorded = sum(b * (s.vocab_size * 4 + (3 * widest + 8 * s.hidden_size) * item) + (64 << 20) for b in buckets)
+        # and every recorded short step of any make: its tokens' activations and its requests' logits
+        if graph_rows and graph_tokens:
+            for t in self._token_bucket_sizes(graph_tokens):
+                for b in [b for b in (1, 4, 16) if b < graph_rows] + [graph_rows]:
+                    recorded += t * (3 * widest + 8 * s.hidden_size) * item + b * s.vocab_size * 4 + (32 << 20)
         budget = total * utilization - (total - free) - activations - recorded
         pages = int(budget // page_bytes)
         if pages <= 0:
             raise RuntimeError(f"no memory left for the cache: {free / 2**30:.1f} GiB free of {total / 2**30:.1f}, "
                                f"one page needs {page_bytes / 2**20:.1f} MiB")
         return pages
+
+    @staticmethod
+    def _token_bucket_sizes(largest: int) -> list[int]:
+        """Token counts that have a recorded short step: powers of two from 16 on, up to ``largest``."""
+        return [t for t in (16, 32, 64, 128, 256, 512, 1024, 2048) if t < largest] + [largest] if largest else []
 
     @staticmethod
     def _bucket_sizes(largest: int) -> list[int]:
@@ -227,7 +247,8 @@ class ModelRunner:
             offset += n
         return out
 
-    def _layout(self, entries: list[StepEntry], pad_to: int | None = None, table_width: int | None = None):
+    def _layout(self, entries: list[StepEntry], pad_to: int | None = None, table_width: int | None = None,
+                pad_tokens_to: int | None = None):
         """Reserves pages and lays the batch out as int32 arrays on the host.
         ``pad_to``: number of requests the arrays are made for (a graph's bucket; only for
         single-token entries): the padding rows store nothing and their results are dropped.
@@ -272,11 +293,17 @@ class ModelRunner:
                                  f"{cache.num_free_pages(gi)} are free")
         if new_requests > cache.num_free_slots():
             raise OutOfPages(f"the step brings {new_requests} new requests, {cache.num_free_slots()} state slots are free")
+        if pad_tokens_to is not None:
+            return self._layout_general(entries, pad_to, table_width, pad_tokens_to)
         if all(len(e.tokens) == 1 for e in entries):
             return self._layout_single_tokens(entries, pad_to, table_width)
         return self._layout_general(entries, pad_to, table_width)
 
-    def _layout_general(self, entries: list[StepEntry], pad_to: int | None, table_width: int | None):
+    def _layout_general(self, entries: list[StepEntry], pad_to: int | None, table_width: int | None,
+                        pad_tokens_to: int | None = None):
+        """``pad_to`` requests of one token each fill the batch (a graph of single tokens); or, with ``pad_tokens_to``
+        (a graph of a short step of any make), ``pad_to`` requests without tokens and one more that owns the
+        ``pad_tokens_to - T`` tokens which fill the bucket."""
         cache = self.cache
         starts, new_lens = [], []
         for e in entries:
@@ -290,15 +317,21 @@ class ModelRunner:
 
         B = len(entries)
         pad = 0 if pad_to is None else pad_to - B
-        q_lens = np.array([len(e.tokens) for e in entries] + [1] * pad, dtype=np.int32)
+        real_tokens = sum(len(e.tokens) for e in entries)
+        if pad_tokens_to is None:
+            pad_q = [1] * pad
+        else:
+            pad_q = [0] * pad + [pad_tokens_to - real_tokens]
+            pad += 1
+        q_lens = np.array([len(e.tokens) for e in entries] + pad_q, dtype=np.int32)
         T = int(q_lens.sum())
         cu = np.zeros(B + pad + 1, dtype=np.int32)
         np.cumsum(q_lens, out=cu[1:])
-        input_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries] + [np.zeros(pad, np.int32)])
+        input_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries] + [np.zeros(T - real_tokens, np.int32)])
         token_req = np.repeat(np.arange(B + pad, dtype=np.int32), q_lens)
         positions = (np.arange(T, dtype=np.int32) - np.repeat(cu[:-1], q_lens)
                      + np.repeat(np.array(starts + [0] * pad, dtype=np.int32), q_lens))
-        context_lens = np.array(new_lens + [1] * pad, dtype=np.int32)
+        context_lens = np.array(new_lens + pad_q, dtype=np.int32)
         # (padding rows work on the spare row of the state pools)
         state_slots = np.array([cache.state_slot(e.request_id) for e in entries] + [self.num_state_slots] * pad,
                                dtype=np.int32)
@@ -308,9 +341,12 @@ class ModelRunner:
         for gi, g in enumerate(cache.groups):
             tables = [cache.block_table(e.request_id, gi) for e in entries]
             width = table_width or max(1, max(len(t) for t in tables))
-            # padding rows read their one key on the spare page (zeros) and store nothing (slot -1)
+            # padding rows read their keys on the spare page (zeros) and store nothing (slot -1)
             bt = np.full((B + pad, width), NO_PAGE, dtype=np.int32)
-            bt[B:, 0] = self.num_pages
+            if pad_tokens_to is None:
+                bt[B:, 0] = self.num_pages
+            else:
+                bt[-1, :max(1, -(-int(pad_q[-1]) // g.page_size))] = self.num_pages
             slot_mapping = np.full(T, -1, dtype=np.int32)
             for i, t in enumerate(tables):
                 ta = np.asarray(t, dtype=np.int32)
@@ -400,6 +436,14 @@ class ModelRunner:
             bucket = next(b for b in self.graph_buckets if b >= len(entries))
             if self._graphs.get(bucket, ...) is not None:
                 return self._graph_step(entries, bucket, keep)
+        elif self.max_graph_tokens and len(entries) <= self.max_graph_batch and all(len(e.want) <= 1 for e in entries):
+            tokens = sum(len(e.tokens) for e in entries)
+            width = -(-self.max_model_len // self.page_size)
+            if tokens <= self.max_graph_tokens and self.max_graph_tokens <= width * self.page_size:
+                key = (next(t for t in self.mixed_token_buckets if t >= tokens),
+                       next(b for b in self.mixed_request_buckets if b >= len(entries)))
+                if self._mixed_graphs.get(key, ...) is not None:
+                    return self._mixed_graph_step(entries, key, keep)
         ctx, new_lens = self.build_context(entries)
         if self.device.type == "cuda":
             from ..native import ops
@@ -448,6 +492,38 @@ class ModelRunner:
         if rows == list(range(len(entries))):
             return g["logits"][:len(entries)].clone() if keep else g["logits"][:len(entries)]
         return g["logits"][torch.tensor(rows, device=self.device)]
+
+    def _mixed_graph_step(self, entries: list[StepEntry], key: tuple[int, int], keep: bool = True) -> torch.Tensor | None:
+        """A short step of any make: padded to the bucket (tokens, requests), written into the bucket's fixed index
+        buffer, and the bucket's graph is replayed. One graph serves every context length: nothing in such a step is
+        laid out for the lengths (the attention of prompt portions takes its bounds from the device)."""
+        token_bucket, request_bucket = key
+        width = -(-self.max_model_len // self.page_size)
+        arrays, meta = self._layout(entries, pad_to=request_bucket, table_width=width, pad_tokens_to=token_bucket)
+        # the places whose logits are wanted, one row per request of the bucket (unused rows repeat row 0)
+        rows = meta["rows"]
+        arrays.append(np.array(rows + [0] * (request_bucket - len(rows)), dtype=np.int32))
+        g = self._mixed_graphs.get(key)
+        if g is None:
+            g = self._capture_mixed(key, arrays, meta, width, len(rows))
+            self._mixed_graphs[key] = g if g["graph"] is not None else None
+        if g["graph"] is not None:
+            g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
+            self._copy_issued()
+            g["graph"].replay()
+        for e, n in zip(entries, meta["new_lens"]):
+            self._poison(self.cache.commit(e.request_id, n, e.tokens))
+        if not rows:
+            return None
+        return g["logits"][:len(rows)].clone() if keep else g["logits"][:len(rows)]
+
+    def _capture_mixed(self, key: tuple[int, int], arrays: list[np.ndarray], meta: dict, width: int, num_real: int) -> dict:
+        index, dev = self._index_buffer(arrays)
+        token_bucket, request_bucket = key
+        meta = dict(meta, max_q_len=token_bucket)            # (the launch is made for the longest portion the bucket can hold)
+        ctx = self._context(dev[:-1], meta, dev[-1], request_bucket, max_context_len=width * self.page_size)
+        graph, logits = self._record(ctx, f"{token_bucket} tokens of {request_bucket} requests", num_real, planned=0)
+        return {"graph": graph, "index": index, "logits": logits, "ctx": ctx}
 
     # ------------------------------------------------------------------ a decoding step issued ahead of its tokens
     def can_step_ahead(self, request_ids: list) -> bool:
@@ -520,31 +596,41 @@ class ModelRunner:
                 for name, t in pool.items():
                     t[slots_t] = kept[name][rows_t]
 
-    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int, num_real: int) -> dict:
-        """Runs the bucket's step once eagerly on its fixed buffers (so that every kernel library is loaded
-        and the allocator is warm), then records it, and checks the graph if a library call went into it.
-        A model with per-request state is stepped several times here on the same tokens: the state that the
-        step found is put back before each run, so that all of them, and the caller's, start from it."""
-        from ..native import ops
+    def _index_buffer(self, arrays: list[np.ndarray]) -> tuple[torch.Tensor, list[torch.Tensor]]:
+        """A graph's fixed buffer of index arrays, filled with these, and the views of the arrays in it."""
         sizes = [a.size for a in arrays]
         index = torch.zeros(sum(sizes), dtype=torch.int32, device=self.device)
-        host = torch.from_numpy(np.concatenate([a.reshape(-1) for a in arrays]))
-        index.copy_(host)
+        index.copy_(torch.from_numpy(np.concatenate([a.reshape(-1) for a in arrays])))
         dev, offset = [], 0
         for a, n in zip(arrays, sizes):
             dev.append(index[offset:offset + n].view(a.shape))
             offset += n
+        return index, dev
+
+    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int, num_real: int) -> dict:
+        """The graph of a step of single tokens for ``bucket`` requests."""
+        index, dev = self._index_buffer(arrays)
         all_rows = torch.arange(bucket, dtype=torch.int32, device=self.device)
         ctx = self._context(dev, meta, all_rows, bucket, max_context_len=width * self.page_size)
+        # the graph's launches are fixed: kernels that split the keys plan for this step's longest context (replays
+        # with other lengths stay right: the block tables and the splits' results are made for max_model_len)
+        planned = max(256, meta["max_context_len"])
+        graph, logits = self._record(ctx, f"{bucket} requests", num_real, planned)
+        return {"graph": graph, "index": index, "logits": logits, "ctx": ctx, "planned": planned}
+
+    def _record(self, ctx: StepContext, what: str, num_real: int, planned: int):
+        """Runs the step of ``ctx`` once eagerly on its fixed buffers (so that every kernel library is loaded
+        and the allocator is warm), then records it, and checks the graph if a library call went into it. Returns
+        (graph, its logits), or (None, the eager step's logits) if the step cannot be recorded or its graph fails.
+        A model with per-request state is stepped several times here on the same tokens: the state that the
+        step found is put back before each run, so that all of them, and the caller's, start from it."""
+        from ..native import ops
         backend = ops.backend()
         with_library = self.dtype == torch.bfloat16           # (the float32 path has kernels of its own throughout)
         old = (getattr(backend, "own_kernels_only", False), getattr(backend, "planned_context", 0),
                getattr(backend, "measure_linears", False))
         backend.own_kernels_only = False
         backend.measure_linears = True                        # few-rows products of new shapes are timed both ways, once
-        # the graph's launches are fixed: kernels that split the keys plan for this step's longest context (replays
-        # with other lengths stay right: the block tables and the splits' results are made for max_model_len)
-        planned = max(256, meta["max_context_len"])
         backend.planned_context = planned
         state_slots = ctx.state_slots.long()
         found = [{name: t[state_slots] for name, t in pool.items()} for pool in self.state_pools]
@@ -563,9 +649,9 @@ class ModelRunner:
                 with torch.cuda.graph(graph):
                     logits = self.model.logits(self.model.forward(ctx))
             except RuntimeError as err:                       # something in the step cannot be recorded
-                print(f"[nanohybrid_vlm_amd] no graph for {bucket} requests ({str(err).splitlines()[0][:200]}); "
+                print(f"[nanohybrid_vlm_amd] no graph for {what} ({str(err).splitlines()[0][:200]}); "
                       "steps of this size run eagerly", file=sys.stderr, flush=True)
-                return {"graph": None, "index": index, "logits": eager, "ctx": ctx, "planned": planned}
+                return None, eager
             if with_library or self.state_pools:
                 for _ in range(3):
                     logits.fill_(float("nan"))
@@ -574,9 +660,9 @@ class ModelRunner:
                     torch.cuda.synchronize()
                     # (the rows of the requests: what the padding rows hold is nobody's result)
                     if not self.graph_check(logits[:num_real], eager[:num_real]):
-                        print(f"[nanohybrid_vlm_amd] the graph for {bucket} requests differs from the eager step when "
+                        print(f"[nanohybrid_vlm_amd] the graph for {what} differs from the eager step when "
                               "replayed; steps of this size run eagerly", file=sys.stderr, flush=True)
-                        return {"graph": None, "index": index, "logits": eager, "ctx": ctx, "planned": planned}
+                        return None, eager
                     put_state_back()
                     self.model.logits(self.model.forward(ctx))      # eager work between the replays
                     torch.cuda.synchronize()
@@ -585,7 +671,7 @@ class ModelRunner:
             backend.own_kernels_only, backend.planned_context, backend.measure_linears = old
             if hasattr(backend, "end_measurements"):
                 backend.end_measurements()
-        return {"graph": graph, "index": index, "logits": logits, "ctx": ctx, "planned": planned}
+        return graph, logits
 
     def get_memory_stats(self) -> dict:
         """Bytes of weights, cache and state pools, pages per group, and the allocator's and the device's view
@@ -609,6 +695,8 @@ class ModelRunner:
             "graphs_recorded": sorted(b for b, g in self._graphs.items() if g is not None),
             "graphs_refused": sorted(b for b, g in self._graphs.items() if g is None),
             "graphs_rerecorded": self.graphs_rerecorded,
+            "mixed_graphs_recorded": sorted(k for k, g in self._mixed_graphs.items() if g is not None),
+            "mixed_graphs_refused": sorted(k for k, g in self._mixed_graphs.items() if g is None),
         }
         if self.device.type == "cuda":
             free, total = torch.cuda.mem_get_info(self.device)

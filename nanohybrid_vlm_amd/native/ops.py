@@ -284,8 +284,8 @@ class NativeBackend:
             if step != self.step_number:                     # (a model's layers meet the same shape in one step)
                 met += 1
                 self._met[key] = (met, self.step_number)
-            if not self.measure_many_rows or met < 3:
-                return None
+            if not self.measure_many_rows or (met < 3 and not self.measure_linears):
+                return None                                  # (before a graph is recorded every new shape is measured at once)
         elif not self.measure_linears:
             return None
         try:

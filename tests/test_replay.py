@@ -455,3 +455,58 @@ def test_trace_run_program_with_a_whole_trace(model_folders, dtype, tmp_path):
                           capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-3000:]
     assert sorted(os.listdir(out_dir), key=lambda n: int(n.split(".")[0])) == [f"{i}.f32" for i in range(len(steps))]
+
+
+# ---------------------------------------------------------------- short steps of any make as graphs
+
+def _last_places_only(steps):
+    """The same steps, asking for one place of every entry (its last): what a serving engine asks for."""
+    return [dict(st, entries=[dict(e, want=[len(e["tokens"]) - 1]) for e in st["entries"]]) for st in steps]
+
+
+def _replay_short_steps(folder, dtype, device, graphs, max_graph_tokens=64):
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    cfg, _ = plain.read_model_folder(folder)
+    requests = _requests(cfg["vocab_size"])
+    full = _plain_logits(folder, requests)
+    results, stats = {}, {"mixed_graphs_recorded": [], "mixed_graphs_refused": []}
+    for mode, steps in [("portions", rc.portions(requests)), ("mixed", rc.mixed(requests))]:
+        steps = _last_places_only(steps)
+        # the plain logits at the places that the steps ask for, request by request
+        want, fed = {}, {rid: 0 for rid in requests}
+        for st in steps:
+            for e in st["entries"]:
+                fed[e["id"]] += len(e["tokens"])
+                want.setdefault(e["id"], []).append(full[e["id"]][fed[e["id"]] - 1])
+        want = {rid: torch.stack(rows) for rid, rows in want.items()}
+        pages = rc.peak_tokens(steps, 8) // 8
+        runner = _poisoned(ModelRunner(folder, dtype=dtype, device=device, page_size=8, num_pages=pages, num_state_slots=4,
+                                       use_graphs=graphs, max_model_len=160, poison_freed_pages=True,
+                                       max_graph_tokens=max_graph_tokens))
+        results[mode] = rc.run_in_process(runner, steps)
+        _check(results[mode], want, tolerance_for(dtype, want), f"{dtype} {mode}, one place a request")
+        for key in stats:
+            stats[key] = sorted(set(stats[key]) | set(runner.get_memory_stats()[key]))
+    return results, stats
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_short_steps_replay_graphs(model_folders, name, dtype):
+    """Portions of prompts, alone and beside decoded tokens, of up to 64 tokens a step: recorded for (tokens,
+    requests) rounded up, the bucket filled by a request of its own on the spare page. The same logits as run
+    eagerly, bit for bit in float32."""
+    folder = model_folders[name]
+    with_graphs, stats = _replay_short_steps(folder, dtype, "cuda:0", graphs=True)
+    assert stats["mixed_graphs_refused"] == [] and len(stats["mixed_graphs_recorded"]) >= 3, stats
+    assert {t for t, _ in stats["mixed_graphs_recorded"]} <= {16, 32, 64}
+    eager, none = _replay_short_steps(folder, dtype, "cuda:0", graphs=False)
+    assert none["mixed_graphs_recorded"] == []
+    for mode in with_graphs:
+        for rid in with_graphs[mode]:
+            if dtype == "float32":
+                assert torch.equal(with_graphs[mode][rid], eager[mode][rid]), f"{mode}: request {rid}"
+            else:
+                d = max_abs_diff(with_graphs[mode][rid], eager[mode][rid])
+                assert d <= 0.5 * TOLERANCE["bfloat16"], f"{mode}: request {rid}: {d:.3e}"
