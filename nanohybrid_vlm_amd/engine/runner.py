@@ -438,11 +438,11 @@ class ModelRunner:
                 return self._graph_step(entries, bucket, keep)
         elif self.max_graph_tokens and len(entries) <= self.max_graph_batch and all(len(e.want) <= 1 for e in entries):
             tokens = sum(len(e.tokens) for e in entries)
-            width = -(-self.max_model_len // self.page_size)
-            if tokens <= self.max_graph_tokens and self.max_graph_tokens <= width * self.page_size:
+            if tokens <= self.max_graph_tokens:
                 key = (next(t for t in self.mixed_token_buckets if t >= tokens),
                        next(b for b in self.mixed_request_buckets if b >= len(entries)))
-                if self._mixed_graphs.get(key, ...) is not None:
+                # (the tokens that fill a bucket stand at positions below the bucket's size: the model must have them)
+                if key[0] <= self.max_model_len and self._mixed_graphs.get(key, ...) is not None:
                     return self._mixed_graph_step(entries, key, keep)
         ctx, new_lens = self.build_context(entries)
         if self.device.type == "cuda":

@@ -510,3 +510,23 @@ def test_short_steps_replay_graphs(model_folders, name, dtype):
             else:
                 d = max_abs_diff(with_graphs[mode][rid], eager[mode][rid])
                 assert d <= 0.5 * TOLERANCE["bfloat16"], f"{mode}: request {rid}: {d:.3e}"
+
+
+@pytest.mark.gpu
+def test_short_step_graphs_stay_within_the_models_positions(model_folders):
+    """The tokens that fill a bucket stand at positions below the bucket's size; a model that is allowed fewer
+    positions than that runs such steps eagerly."""
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    folder = model_folders["A"]
+    cfg, w = plain.read_model_folder(folder)
+    tokens = rc.random_tokens(cfg["vocab_size"], 40, 5)
+    runner = ModelRunner(folder, dtype="float32", page_size=64, num_pages=2, num_state_slots=2, use_graphs=True,
+                         max_model_len=48, max_graph_tokens=256)
+    got = rc.run_in_process(runner, [{"step": 0, "entries": [{"id": "a", "tokens": tokens, "want": [39]}], "end": ["a"]}])
+    assert runner.get_memory_stats()["mixed_graphs_recorded"] == []           # 40 tokens round up to 64 > 48 positions
+    assert max_abs_diff(got["a"], plain.logits(cfg, w, tokens)[39:]) <= tolerance_for("float32", got)
+    runner = ModelRunner(folder, dtype="float32", page_size=64, num_pages=2, num_state_slots=2, use_graphs=True,
+                         max_model_len=64, max_graph_tokens=256)
+    got = rc.run_in_process(runner, [{"step": 0, "entries": [{"id": "a", "tokens": tokens, "want": [39]}], "end": ["a"]}])
+    assert runner.get_memory_stats()["mixed_graphs_recorded"] == [(64, 1)]
+    assert max_abs_diff(got["a"], plain.logits(cfg, w, tokens)[39:]) <= tolerance_for("float32", got)
