@@ -199,8 +199,10 @@ class ModelRunner:
 
     @staticmethod
     def _token_bucket_sizes(largest: int) -> list[int]:
-        """Token counts that have a recorded short step: powers of two from 16 on, up to ``largest``."""
-        return [t for t in (16, 32, 64, 128, 256, 512, 1024, 2048) if t < largest] + [largest] if largest else []
+        """Token counts that have a recorded short step: powers of two from 16 on and the sizes half way between, up to
+        ``largest`` (a step is padded to the next one: at the 8B shape a token of padding costs about 13 us)."""
+        sizes = sorted({t for p in range(4, 24) for t in (1 << p, 3 << p >> 1)})
+        return [t for t in sizes if t < largest] + [largest] if largest else []
 
     @staticmethod
     def _bucket_sizes(largest: int) -> list[int]:
