@@ -50,7 +50,7 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--block-size", type=int, default=256, help="tokens per page of the cache")
     ap.add_argument("--num-blocks", type=int, default=-1, help="pages of the cache (-1: from free memory)")
     ap.add_argument("--max-num-seqs", type=int, default=512)
-    ap.add_argument("--max-graph-batch", type=int, default=64, help="decode steps of up to this many requests replay a graph")
+    ap.add_argument("--max-graph-batch", type=int, default=256, help="decode steps of up to this many requests replay a graph")
     ap.add_argument("--max-graph-tokens", type=int, default=256,
                     help="other steps (prompt portions, alone or beside decoded tokens) of up to this many tokens replay a graph; 0: none")
     ap.add_argument("--no-run-ahead", action="store_true",

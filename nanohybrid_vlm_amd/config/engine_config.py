@@ -23,7 +23,7 @@ class EngineConfig:
     max_model_len: int = 4096                   # capped by max_position_embeddings
     gpu_memory_utilization: float = 0.9
     enforce_eager: bool = False                 # True: no HIP graphs for decode
-    max_graph_batch: int = 64                   # decode steps of up to this many requests replay a graph
+    max_graph_batch: int = 256                  # decode steps of up to this many requests replay a graph
     max_graph_tokens: int = 256                 # so do other steps (prompt portions, alone or beside decoded tokens) of up to this many tokens; 0: none
     run_ahead: bool = True                      # a decode step that is bound to follow is issued before the host knows the tokens it feeds
     eos: int = -1                               # filled from config.json when -1

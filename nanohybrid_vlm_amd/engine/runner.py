@@ -105,7 +105,7 @@ class ModelRunner:
         # stores nothing, and the requests that fill it have no tokens. 0 switches this off.
         self.max_graph_tokens = max_graph_tokens if self.use_graphs else 0
         self.mixed_token_buckets = self._token_bucket_sizes(self.max_graph_tokens)
-        self.mixed_request_buckets = [b for b in (1, 4, 16) if b < max_graph_batch] + [max_graph_batch]
+        self.mixed_request_buckets = [b for b in (1, 4, 16, 64) if b < max_graph_batch] + [max_graph_batch]
         self._mixed_graphs: dict[tuple[int, int], dict | None] = {}
         self.graph_check = torch.equal                # (replay, eager) -> bool; a test replaces it to force a refusal
         self.graphs_rerecorded = 0                    # graphs recorded again because the contexts had outgrown their layout
@@ -188,7 +188,7 @@ class ModelRunner:
         # and every recorded short step of any make: its tokens' activations and its requests' logits
         if graph_rows and graph_tokens:
             for t in self._token_bucket_sizes(graph_tokens):
-                for b in [b for b in (1, 4, 16) if b < graph_rows] + [graph_rows]:
+                for b in [b for b in (1, 4, 16, 64) if b < graph_rows] + [graph_rows]:
                     recorded += t * (3 * widest + 8 * s.hidden_size) * item + b * s.vocab_size * 4 + (32 << 20)
         budget = total * utilization - (total - free) - activations - recorded
         pages = int(budget // page_bytes)
