@@ -53,6 +53,8 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--max-graph-batch", type=int, default=256, help="decode steps of up to this many requests replay a graph")
     ap.add_argument("--max-graph-tokens", type=int, default=256,
                     help="other steps (prompt portions, alone or beside decoded tokens) of up to this many tokens replay a graph; 0: none")
+    ap.add_argument("--warm-up", action="store_true",
+                    help="measure the matrix products and record the graphs of every step size when the engine starts")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="every step is issued only when the tokens of the step before are known to the host")
     ap.add_argument("--max-model-len", type=int, default=4096)
@@ -107,7 +109,7 @@ def _make_llm(args):
                max_num_batched_tokens=args.token_budget, gpu_memory_utilization=args.gpu_memory_utilization,
                kvcache_block_size=args.block_size, num_kvcache_blocks=args.num_blocks, max_num_seqs=args.max_num_seqs,
                max_model_len=args.max_model_len, scheduler_policy=args.scheduler_policy, seed=args.seed,
-               enable_prefix_cache=args.enable_prefix_cache, max_graph_batch=args.max_graph_batch, max_graph_tokens=args.max_graph_tokens,
+               enable_prefix_cache=args.enable_prefix_cache, max_graph_batch=args.max_graph_batch, max_graph_tokens=args.max_graph_tokens, warm_up=args.warm_up,
                run_ahead=not args.no_run_ahead, gemm_choices=args.gemm_choices, measure_gemms=not args.no_measure_gemms,
                residual_dtype=args.residual_dtype)
 

@@ -25,6 +25,7 @@ class EngineConfig:
     enforce_eager: bool = False                 # True: no HIP graphs for decode
     max_graph_batch: int = 256                  # decode steps of up to this many requests replay a graph
     max_graph_tokens: int = 256                 # so do other steps (prompt portions, alone or beside decoded tokens) of up to this many tokens; 0: none
+    warm_up: bool = False                       # True: every size of step that replays a graph is met once when the engine starts
     run_ahead: bool = True                      # a decode step that is bound to follow is issued before the host knows the tokens it feeds
     eos: int = -1                               # filled from config.json when -1
     kvcache_block_size: int = 256               # tokens in a page (any positive number)

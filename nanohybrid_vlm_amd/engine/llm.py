@@ -144,6 +144,8 @@ class LLM:
         self._completed_metrics: list[RequestMetrics] = []
         self._ahead = None               # a decoding step issued before its tokens were known to the host (see step)
         self.num_steps_ahead = 0         # steps that were already under way when their turn came
+        if cfg.warm_up:
+            self.warm_up()
 
     # ------------------------------------------------------------------ how matrix products are done
     @staticmethod
@@ -179,6 +181,34 @@ class LLM:
         with open(path, "w") as f:
             json.dump(self.gemm_choices(), f, indent=1, sort_keys=True)
         return path
+
+    # ------------------------------------------------------------------ before the first request
+    def warm_up(self, batch_sizes=None, token_counts=None) -> dict:
+        """Meets every size of step that replays a graph once, before any request does: the matrix products of each
+        size are measured (which is what takes the time: a fraction of a second a size) and the graphs of single-token
+        steps (for short contexts; one for longer contexts is recorded when they are met, without measuring again)
+        and of short steps of any other make are recorded. The reference records its graphs when the engine starts
+        (nanovllm/engine/model_runner.py:2559-2594); here it is asked for: engine option ``warm_up``, or this call.
+        ``batch_sizes``, ``token_counts``: the sizes to meet (default: all that the engine's limits allow).
+        Returns what was recorded. Nothing of it stays in the cache."""
+        runner = self.runner
+        if not runner.use_graphs or self.scheduler.running or self.scheduler.waiting:
+            return {"graphs_recorded": [], "mixed_graphs_recorded": []}
+        most = min(self.config.max_num_seqs, runner.cache.num_free_slots(), runner.num_pages)
+        sizes = [b for b in (batch_sizes or runner.graph_buckets) if b <= most]
+        for b in sizes:
+            ids = [("warm up", i) for i in range(b)]
+            runner.step([StepEntry(r, [0], []) for r in ids])              # a first token each, then a step of single tokens
+            runner.step([StepEntry(r, [0], [0]) for r in ids])
+            for r in ids:
+                runner.finish(r)
+        counts = token_counts if token_counts is not None else runner.mixed_token_buckets
+        for t in counts:
+            if t <= min(runner.max_graph_tokens, runner.max_model_len, runner.num_pages * runner.page_size):
+                runner.step([StepEntry(("warm up", 0), [0] * t, [t - 1])])
+                runner.finish(("warm up", 0))
+        stats = runner.get_memory_stats()
+        return {key: stats[key] for key in ("graphs_recorded", "mixed_graphs_recorded")}
 
     # ------------------------------------------------------------------ requests
     def add_request(self, prompt, sampling_params: SamplingParams | None = None) -> int:

@@ -370,3 +370,26 @@ def test_pinned_gemm_choices_make_bfloat16_runs_repeat_bit_for_bit(model_folders
     assert torch.equal(again, measured)
     backend.measuring_allowed = True
     backend.chosen.clear()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_warm_up_records_the_graphs_ahead(model_folders, dtype):
+    """With ``warm_up`` every size of step that replays a graph is met once when the engine starts: the graphs are
+    there before the first request, nothing stays in the cache, and generation gives the plain tokens."""
+    folder = model_folders["B"]
+    cfg, w = plain.read_model_folder(folder)
+    llm = LLM(folder, dtype=dtype, kvcache_block_size=16, num_kvcache_blocks=40, max_num_seqs=8, max_graph_tokens=64,
+              max_num_batched_tokens=64, warm_up=True)
+    stats = llm.get_memory_stats()
+    assert stats["graphs_recorded"] == [1, 2, 3, 4, 6, 8] and stats["graphs_refused"] == []
+    assert stats["mixed_graphs_recorded"] == [(16, 1), (24, 1), (32, 1), (48, 1), (64, 1)] and stats["mixed_graphs_refused"] == []
+    assert stats["live_requests"] == 0 and stats["groups"][0]["free_pages"] == 40
+    llm.runner.cache.check()
+    if dtype == "float32":
+        prompts = [random_tokens(cfg["vocab_size"], n, 300 + n) for n in (5, 30, 47, 12)]
+        sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+        out = llm.generate(prompts, sp)
+        assert [o["token_ids"] for o in out] == [plain.greedy_generate(cfg, w, p, 6) for p in prompts]
+    # asked for again, and with requests under way, it does nothing
+    assert llm.warm_up(batch_sizes=[1], token_counts=[16])["graphs_recorded"] == [1, 2, 3, 4, 6, 8]
