@@ -136,9 +136,10 @@ def test_toy_generates_through_the_entry_point_on_gpu(toy_architecture, tmp_path
             # per-request state keeps a model neither out of graphs nor out of steps issued ahead (a step issued
             # ahead may have to be taken back, which a window's pages, given back as it moves, do not allow)
             assert stats["graphs_recorded"] and not stats["graphs_refused"], stats
+            assert stats["mixed_graphs_recorded"] and not stats["mixed_graphs_refused"], stats   # prompt portions as graphs too
             assert (llm.num_steps_ahead > 0) == no_window
         else:
-            assert not stats["graphs_recorded"] and llm.num_steps_ahead == 0
+            assert not stats["graphs_recorded"] and not stats["mixed_graphs_recorded"] and llm.num_steps_ahead == 0
 
 
 @pytest.mark.gpu
