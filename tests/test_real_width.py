@@ -117,6 +117,8 @@ def test_generation_at_real_widths(real_width_folder):
     params = [SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True)] * 4 + [SamplingParams(temperature=0.8, max_tokens=8, seed=3)]
     outs = llm.generate(prompts, params, use_tqdm=False)
     assert llm.num_steps_ahead > 0
+    stats = llm.get_memory_stats()
+    assert stats["mixed_graphs_recorded"] and not stats["mixed_graphs_refused"], stats      # the prompts' portions ran as graphs
     with torch.no_grad():
         for p, o in list(zip(prompts, outs))[:4]:
             ids = list(p)
@@ -127,3 +129,39 @@ def test_generation_at_real_widths(real_width_folder):
     again = LLM(real_width_folder, dtype="bfloat16", kvcache_block_size=256, num_kvcache_blocks=12, max_num_batched_tokens=128,
                 max_model_len=512, run_ahead=False).generate(prompts, params, use_tqdm=False)
     assert [o["token_ids"] for o in again] == [o["token_ids"] for o in outs]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_short_steps_as_graphs_at_real_widths(real_width_folder, plain_on_gpu, dtype):
+    """Portions beside decoded tokens, one wanted place a request: the steps of up to 256 tokens replay graphs whose
+    buckets are filled by a request of their own; the logits are the plain implementation's, and in float32 the
+    eager run's bit for bit."""
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    requests, full = plain_on_gpu
+    steps = rc.mixed(requests, sizes=(100, 7, 64, 2, 129, 33))
+    steps = [dict(st, entries=[dict(e, want=[len(e["tokens"]) - 1]) for e in st["entries"]]) for st in steps]
+    want, fed = {}, {rid: 0 for rid in requests}
+    for st in steps:
+        for e in st["entries"]:
+            fed[e["id"]] += len(e["tokens"])
+            want.setdefault(e["id"], []).append(full[e["id"]][fed[e["id"]] - 1])
+    want = {rid: torch.stack(rows) for rid, rows in want.items()}
+    tol = tolerance_for(dtype, full)
+    results = {}
+    for graphs in (True, False):
+        pages = rc.peak_tokens(steps, 256) // 256
+        runner = ModelRunner(real_width_folder, dtype=dtype, page_size=256, num_pages=pages, num_state_slots=4,
+                             use_graphs=graphs, max_model_len=768, poison_freed_pages=True)
+        for kv in runner.kv_tensors:
+            kv.fill_(float("nan"))
+        results[graphs] = rc.run_in_process(runner, steps)
+        for rid in requests:
+            d = max_abs_diff(results[graphs][rid], want[rid])
+            assert d <= tol, f"{dtype}, graphs {graphs}: request {rid}: max diff {d:.3e} > {tol:.1e}"
+        stats = runner.get_memory_stats()
+        assert bool(stats["mixed_graphs_recorded"]) == graphs and not stats["mixed_graphs_refused"], stats
+        del runner
+        torch.cuda.empty_cache()
+    if dtype == "float32":
+        for rid in requests:
+            assert torch.equal(results[True][rid], results[False][rid]), rid
