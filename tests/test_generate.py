@@ -393,3 +393,45 @@ def test_warm_up_records_the_graphs_ahead(model_folders, dtype):
         assert [o["token_ids"] for o in out] == [plain.greedy_generate(cfg, w, p, 6) for p in prompts]
     # asked for again, and with requests under way, it does nothing
     assert llm.warm_up(batch_sizes=[1], token_counts=[16])["graphs_recorded"] == [1, 2, 3, 4, 6, 8]
+
+
+def _stress(folder, device, seed, options):
+    """Requests of random lengths arrive a few at a time while others decode, with so few pages that some are
+    pushed out and computed again; every request's tokens must be the plain implementation's."""
+    import random
+    rnd_ = random.Random(seed)
+    cfg, w = plain.read_model_folder(folder)
+    V = cfg["vocab_size"]
+    requests = [(random_tokens(V, rnd_.randint(1, 70), 1000 * seed + i), rnd_.randint(1, 18)) for i in range(36)]
+    llm = LLM(folder, dtype="float32", device=device, kvcache_block_size=8, num_kvcache_blocks=rnd_.choice([28, 40, 90]),
+              max_num_batched_tokens=rnd_.choice([16, 48, 96]), max_num_seqs=rnd_.choice([4, 9, 36]),
+              max_model_len=96, max_prefill_wait_ms=rnd_.choice([0.0, 1e9]), **options)
+    ids, done, waiting = {}, {}, list(enumerate(requests))
+    while waiting or not llm.is_finished():
+        for _ in range(rnd_.randint(0, 3)):
+            if waiting:
+                i, (prompt, n) = waiting.pop(0)
+                ids[llm.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True))] = i
+        if not llm.is_finished():
+            done.update(llm.step()[0])
+    got = {ids[sid]: toks for sid, toks in done.items()}
+    for i, (prompt, n) in enumerate(requests):
+        assert got[i] == plain.greedy_generate(cfg, w, prompt, n), f"seed {seed}: request {i}"
+    stats = llm.get_memory_stats()
+    assert stats["live_requests"] == 0 and stats["groups"][0]["free_pages"] == stats["groups"][0]["pages"]
+    llm.runner.cache.check()
+    return llm, stats
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_engine_under_random_arrivals_on_emulated_kernels(model_folders, emulated_kernels, seed):
+    _stress(model_folders["B"], "cpu", seed, {})
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(6))
+def test_engine_under_random_arrivals_on_gpu(model_folders, seed):
+    """The same with recorded steps of both kinds (single tokens; short steps of any make) and steps issued ahead."""
+    llm, stats = _stress(model_folders["B"], "cuda:0", seed, dict(max_graph_tokens=64))
+    assert not stats["graphs_refused"] and not stats["mixed_graphs_refused"]
+    assert stats["graphs_recorded"] and stats["mixed_graphs_recorded"], stats
