@@ -479,7 +479,9 @@ class ModelRunner:
         longest = max(256, meta["max_context_len"])
         if g is None or not g["planned"] // 2 < longest <= g["planned"] + g["planned"] // 2:
             self.graphs_rerecorded += g is not None
-            g = self._capture(bucket, arrays, meta, width, len(entries))
+            # (a graph recorded again holds the same library calls as the one before it, which passed its check:
+            # it is not checked again, and a step that records again takes 4 step times instead of 10)
+            g = self._capture(bucket, arrays, meta, width, len(entries), check=g is None)
             self._graphs[bucket] = g if g["graph"] is not None else None
         if g["graph"] is not None:
             g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
@@ -609,7 +611,7 @@ class ModelRunner:
             offset += n
         return index, dev
 
-    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int, num_real: int) -> dict:
+    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int, num_real: int, check: bool = True) -> dict:
         """The graph of a step of single tokens for ``bucket`` requests."""
         index, dev = self._index_buffer(arrays)
         all_rows = torch.arange(bucket, dtype=torch.int32, device=self.device)
@@ -617,10 +619,10 @@ class ModelRunner:
         # the graph's launches are fixed: kernels that split the keys plan for this step's longest context (replays
         # with other lengths stay right: the block tables and the splits' results are made for max_model_len)
         planned = max(256, meta["max_context_len"])
-        graph, logits = self._record(ctx, f"{bucket} requests", num_real, planned)
+        graph, logits = self._record(ctx, f"{bucket} requests", num_real, planned, check)
         return {"graph": graph, "index": index, "logits": logits, "ctx": ctx, "planned": planned}
 
-    def _record(self, ctx: StepContext, what: str, num_real: int, planned: int):
+    def _record(self, ctx: StepContext, what: str, num_real: int, planned: int, check: bool = True):
         """Runs the step of ``ctx`` once eagerly on its fixed buffers (so that every kernel library is loaded
         and the allocator is warm), then records it, and checks the graph if a library call went into it. Returns
         (graph, its logits), or (None, the eager step's logits) if the step cannot be recorded or its graph fails.
@@ -654,7 +656,7 @@ class ModelRunner:
                 print(f"[nanohybrid_vlm_amd] no graph for {what} ({str(err).splitlines()[0][:200]}); "
                       "steps of this size run eagerly", file=sys.stderr, flush=True)
                 return None, eager
-            if with_library or self.state_pools:
+            if check and (with_library or self.state_pools):
                 for _ in range(3):
                     logits.fill_(float("nan"))
                     put_state_back()
