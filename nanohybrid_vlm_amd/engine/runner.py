@@ -100,7 +100,7 @@ class ModelRunner:
         # Short steps of any make (portions of prompts, beside decoded tokens or alone) are bound by their launches as
         # well: some 350 kernels of a few microseconds each against 15 to 20 us of host work a launch. A step of up to
         # ``max_graph_tokens`` tokens in which every request wants at most one place replays a graph too, recorded for
-        # (tokens, requests) rounded up to the next sizes of ``mixed_token_buckets`` and the decode buckets: the tokens
+        # (tokens, requests) rounded up to the next sizes of ``mixed_token_buckets`` and ``mixed_request_buckets``: the tokens
         # that fill the bucket belong to a request of their own, whose keys are the zeros of the spare page and which
         # stores nothing, and the requests that fill it have no tokens. 0 switches this off.
         self.max_graph_tokens = max_graph_tokens if self.use_graphs else 0
