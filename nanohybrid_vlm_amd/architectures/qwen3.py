@@ -209,6 +209,9 @@ def _shape(layers, hidden, heads, kv_heads, head_dim, inter, vocab=151936, theta
 SHAPES = {
     "tinyA": _shape(2, 64, 4, 2, 16, 128, vocab=256, theta=10000.0, eps=1e-6, tie=True, max_pos=128),
     "tinyB": _shape(3, 96, 6, 1, 32, 160, vocab=389, theta=1000000.0, eps=1e-5, tie=False, max_pos=256),
+    "0.6b": _shape(28, 1024, 16, 8, 128, 3072, tie=True),
+    "1.7b": _shape(28, 2048, 16, 8, 128, 6144, tie=True),
+    "4b": _shape(36, 2560, 32, 8, 128, 9728, tie=True),
     "8b": _shape(36, 4096, 32, 8, 128, 12288),
     "14b": _shape(40, 5120, 40, 8, 128, 17408),
     "32b": _shape(64, 5120, 64, 8, 128, 25600),
