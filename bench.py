@@ -102,7 +102,12 @@ def run_decode(llm, cfg, batch, prompt_tokens, steps, warmup, seed):
     import torch
     from nanohybrid_vlm_amd import SamplingParams
 
-    sp = SamplingParams(temperature=0.0, max_tokens=warmup + steps + 1, ignore_eos=True)
+    # The engine issues a decode step ahead of its tokens: when the warm-up ends, the first timed step's GPU work is
+    # under way already (and done at the synchronisation). So that the timed window still holds exactly ``steps``
+    # steps of GPU work, the requests live one token longer than the timed steps: the last timed step issues its
+    # successor ahead as every other does, and the closing synchronisation waits for it. Without steps issued
+    # ahead the window holds the timed steps' own work. Either way: ``steps`` steps between the two waits.
+    sp = SamplingParams(temperature=0.0, max_tokens=warmup + steps + 2, ignore_eos=True)
     for p in random_prompts(batch, prompt_tokens, cfg.vocab_size, seed):
         llm.add_request(p, sp)
     while llm.scheduler.waiting:                      # all prompts in, nothing timed
@@ -110,6 +115,7 @@ def run_decode(llm, cfg, batch, prompt_tokens, steps, warmup, seed):
     for _ in range(warmup):
         llm.step()
     torch.cuda.synchronize()
+    ahead = llm._ahead is not None                    # the timed GPU steps are then the ones after the host's
     step_ms = []
     t0 = time.perf_counter()
     last = t0
@@ -123,16 +129,16 @@ def run_decode(llm, cfg, batch, prompt_tokens, steps, warmup, seed):
     seconds = time.perf_counter() - t0
     while not llm.is_finished():
         llm.step()
-    mean_context = prompt_tokens + warmup + (steps + 1) / 2.0
+    mean_context = prompt_tokens + warmup + (steps + 1) / 2.0 + (1 if ahead else 0)
     return seconds, mean_context, step_ms
 
 
-def run_prefill(llm, cfg, prompt_tokens, reps=3):
+def run_prefill(llm, cfg, prompt_tokens, reps=5):
     import torch
     from nanohybrid_vlm_amd import SamplingParams
 
     sp = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
-    best = None
+    times = []
     warm = 3                                          # untimed runs: a shape of many rows is measured in the third step that meets it
     for i in range(reps + warm):
         llm.add_request(random_prompts(1, prompt_tokens, cfg.vocab_size, 900 + i)[0], sp)
@@ -143,8 +149,8 @@ def run_prefill(llm, cfg, prompt_tokens, reps=3):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         if i >= warm:
-            best = dt if best is None else min(best, dt)
-    return best
+            times.append(dt)
+    return percentile(times, 0.5)                     # the median of the timed runs
 
 
 def config_of(args, cfg, full_layers, **more):

@@ -40,7 +40,7 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
                     help="instead of --model: random weights of --shape or --config, drawn on the device")
     ap.add_argument("--shape", default="tinyA",
                     help="with --random-weights: a named configuration of a registered architecture "
-                         "(Qwen3: tinyA, tinyB, 8b, 14b, 32b)")
+                         "(an unknown name lists those there are)")
     ap.add_argument("--config", help="with --random-weights: a config.json to take the sizes from, instead of --shape")
     ap.add_argument("--layers", type=int, help="with --random-weights: override num_hidden_layers")
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32", "bf16", "fp32"))
@@ -76,9 +76,8 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
 
 def _import_plugins(names) -> None:
     """Modules that register architectures or parts of their own when imported."""
-    import importlib
-    for name in names or []:
-        importlib.import_module(name)
+    from .config.registry import import_plugins
+    import_plugins(names)
 
 
 def _named_config(args) -> dict:
@@ -127,6 +126,15 @@ def _percentile(values, q):
     k = (len(values) - 1) * q
     lo, hi = int(k), min(int(k) + 1, len(values) - 1)
     return values[lo] + (values[hi] - values[lo]) * (k - lo)
+
+
+def _summary(values) -> dict | None:
+    """mean, p50, p95, p99 and max of a request metric (tests/5090-test-TP2/suite_common.py:29-45)."""
+    values = [float(v) for v in values if v is not None]
+    if not values:
+        return None
+    return {"mean": statistics.fmean(values), "p50": _percentile(values, 0.5), "p95": _percentile(values, 0.95),
+            "p99": _percentile(values, 0.99), "max": max(values)}
 
 
 def cmd_generate(args) -> int:
@@ -201,6 +209,9 @@ def cmd_bench(args) -> int:
                 "ttft_ms_mean": statistics.fmean(m.ttft_ms for m in metrics),
                 "tpot_ms_mean": statistics.fmean(m.tpot_ms for m in metrics if m.tpot_ms is not None) if n_out > 1 else None,
                 "e2e_ms_mean": statistics.fmean(m.e2e_ms for m in metrics),
+                # the requests' distributions (tests/5090-test-TP2/suite_common.py:103-183)
+                "ttft_ms": _summary(m.ttft_ms for m in metrics), "tpot_ms": _summary(m.tpot_ms for m in metrics),
+                "e2e_ms": _summary(m.e2e_ms for m in metrics), "queue_ms": _summary(m.queue_ms for m in metrics),
                 "preemptions": llm.scheduler.num_preemptions,
             })
             print(json.dumps(results[-1]), flush=True)

@@ -42,11 +42,22 @@ class Architecture:
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}
-_LAZY = {
-    # name -> module that registers it on import (nanovllm/models/registry.py:154-159)
-    "Qwen3ForCausalLM": "nanohybrid_vlm_amd.architectures.qwen3",
-}
-_LAZY_MODEL_TYPES = {"qwen3": "Qwen3ForCausalLM"}
+# Modules that register architectures (and parts) when they are imported. The engine's own architectures are such a
+# module like any other, and no name of an architecture stands here: the package ``architectures`` imports every
+# module that lies in its folder. ``import_plugins`` adds to the list (the command line's ``--plugin``).
+_PLUGINS: list[str] = [__name__.rsplit(".", 2)[0] + ".architectures"]
+_imported: set[str] = set()
+
+
+def import_plugins(names=()) -> None:
+    """Imports modules that register architectures or parts of their own; each once."""
+    for name in names or ():
+        if name not in _PLUGINS:
+            _PLUGINS.append(name)
+    for name in list(_PLUGINS):
+        if name not in _imported:
+            _imported.add(name)
+            importlib.import_module(name)
 
 
 def register_architecture(arch: Architecture, replace: bool = False) -> None:
@@ -60,13 +71,13 @@ def unregister_architecture(name: str) -> None:
 
 
 def _get(name: str) -> Architecture | None:
-    if name not in _ARCHITECTURES and name in _LAZY:
-        importlib.import_module(_LAZY[name])
+    import_plugins()
     return _ARCHITECTURES.get(name)
 
 
 def registered_architectures() -> list[str]:
-    return sorted(set(_ARCHITECTURES) | set(_LAZY))
+    import_plugins()
+    return sorted(_ARCHITECTURES)
 
 
 def named_shapes() -> dict[str, dict]:
@@ -94,9 +105,8 @@ def resolve_architecture(raw_config: dict) -> Architecture:
                     f"(it is registered for {list(arch.model_types)})")
             return arch
     if model_type:
+        import_plugins()
         by_type = [a for a in list(_ARCHITECTURES.values()) if model_type in a.model_types]
-        if not by_type and model_type in _LAZY_MODEL_TYPES:
-            by_type = [_get(_LAZY_MODEL_TYPES[model_type])]
         if by_type:
             arch = by_type[0]
             if listed and arch.name not in listed:

@@ -16,20 +16,6 @@
 // key positions. Each split writes its unnormalised output with (maximum, sum) in
 // float; a second kernel merges the splits in rising order. Keys that are not visible
 // are loaded as zeros (the cache's unused slots may hold anything).
-// (Asking for the next round before this one is computed was measured: the second set of
-// registers leaves one wave per SIMD, and that costs more than the overlap gains. So was
-// doing the queries' norm and rotation and the cache write of the new key and value inside
-// this kernel instead of in one of their own: every split's wave then prepares the queries
-// again and waits for those loads before its first product, which gave back 4 of the 6
-// microseconds saved at 8 requests and lost time at 1 and at 64. So were rounds of 64 keys for launches of one
-// wave per SIMD (5 % less time at 1 and 2 requests, more at 4 and above), and values loaded straight into LDS
-// (global_load_lds, read with ds_read_b64_tr_b16 as in the prompt kernel) with the next round's keys and values
-// asked for before this round is computed: 3 to 8 % less time for this kernel, 1 % of a decoding step. And blocks of two
-// or four waves that take a split's rounds in turn and meet in wave 0 at the end, lane by lane, so that longer splits
-// leave fewer partial results to write and to merge for the same number of waves at work: alone, over caches that
-// change from call to call, 10 % less time at 16 and 32 requests of 2,176 keys (four waves on splits of 512 against one
-// wave on splits of 256), nothing at 1, 8 and 64 requests or at 8,192 keys; inside the model's decoding step the same
-// choice took 2 to 5 % more time at 24, 32 and 48 requests.)
 #include "nhv_common.h"
 #include "nhv_no_alloc.h"
 #include <math.h>
@@ -264,7 +250,9 @@ __global__ __launch_bounds__(64 * W) void merge_splits_kernel(const float* __res
   const int t = item / Hq;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int s0 = lo / split_len, s1 = pos / split_len;
+  // (the launch's splits must cover every position; one that they do not cover loses its last keys here rather
+  // than reading past the splits' results)
+  const int s0 = lo / split_len, s1 = min(pos / split_len, n_splits - 1);
   const float* ml = part_ml + (size_t)item * n_splits * 2;
   float m = -INFINITY;
   for (int s = s0 + lane; s <= s1; s += 64) m = fmaxf(m, ml[s * 2]);
@@ -409,6 +397,11 @@ static int scratch_address(float** ptr) {
 }
 
 extern "C" size_t nhv_decode_attention_no_alloc_limit() { return NHV_NO_ALLOC_SCRATCH_BYTES; }
+
+extern "C" int nhv_decode_attention_no_alloc_init() {
+  float* base = nullptr;
+  return scratch_address(&base);
+}
 
 extern "C" int nhv_decode_attention_bf16_no_alloc(const void* q, const void* k_cache, const void* v_cache, void* out,
                                                   const void* token_req, const void* positions,

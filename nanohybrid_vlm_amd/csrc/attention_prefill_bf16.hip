@@ -32,51 +32,6 @@
 // window + 1 with a window, else 0). Keys outside the block's range are replaced by the
 // nearest key inside it (their P is 0): unused cache slots may hold anything, and 0 * NaN
 // would poison the sums.
-//
-// Measured and not kept: a software pipeline over tiles of 32 keys in four LDS buffers, where one piece of straight
-// code takes tile i + 1's scores, tile i's softmax (against the old references; redone when a row grows) and tile
-// i - 1's P V, so that matrix, vector and LDS instructions of one wave interleave (the compiler did interleave them).
-// It needs about 335 registers: with one wave per SIMD it reached 550 TFLOP/s where this kernel reaches 630 (8,192
-// tokens), held to two waves per SIMD it spills (250). With one wave per SIMD that loop ran at 1,280 TFLOP/s with
-// its matrix instructions alone, 860 with the LDS reads, 900 with the exponentials, 760 with both, and 500-550 with
-// the loads into LDS and the barrier of each tile. More waves do not help either: one row tile a wave, tiles of
-// 32 keys and four waves per SIMD (128 registers, 36 KB of LDS a block) reached 550 TFLOP/s, since every wave then
-// reads all keys and values from LDS for half as many rows.
-//
-// Where the time goes (counters of one run of 8,192 new tokens, 32 query and 8 key/value heads of 128): the matrix
-// cores are busy 36 % of the time; a wave issues 198 other vector instructions for every 64 matrix instructions of a
-// tile (332 before the mask became a compile-time choice and the rescaling a real branch: that change alone took the
-// kernel from 806 to 943 TFLOP/s at 8,192 tokens and from 441 to 537 at 2,048, bit for bit the same results), 67
-// scalar ones and 49 reads of LDS. With the loads of all tiles but the first left out (wrong results, timing only) the
-// kernel takes 16 % less time, without the barriers as well 20 % less: four fifths of the time is the tiles'
-// arithmetic itself, in which the matrix instructions of one wave and the vector instructions of the other on the
-// same SIMD overlap only in part (a microbenchmark: 8 matrix and 24 multiply-add instructions interleaved in one
-// wave take 222 clocks where they take 153 and 148 apart). Measured and not kept after that: the rows' sums of P
-// taken by the matrix cores (a V^T operand of ones; 32 additions fewer and 4 matrix instructions more a tile): 2 %;
-// the tiles' loads as buffer loads whose address is a scalar descriptor and a 32-bit offset (no 64-bit vector
-// additions): nothing; two groups of four waves a block that take the block's key tiles in turn and add up through
-// LDS at the end, so that a block's chain of tiles is half as long (one block of eight waves a compute unit): 3 to
-// 15 % more time at every length, since both groups then wait for their loads at the same moments, which two
-// independent blocks on a compute unit do not; blocks of eight waves with one row tile each, four buffers of tiles
-// and loads three tiles ahead, one block a compute unit: the same 2,048-token time and 15 to 25 % more at 3,072
-// tokens and beyond (every wave reads every tile's keys and values from LDS whatever its number of rows: 256 KB
-// a tile for eight waves, which is what such a block's tile then takes); the reads from LDS written one operand
-// ahead of the products that use them, with and without the order pinned by scheduler group barriers: nothing.
-// Two further attempts, both giving the same bits as this kernel and neither kept. The exponentials of a 16-key
-// sub-tile taken against the references as they stand, right behind its matrix instructions and issued in turn with
-// those of the next sub-tile (the order pinned by scheduler group barriers; a tile in which a row grows is done again
-// the plain way): 8 to 10 % more time at every length, with the order pinned or left to the compiler. And blocks of
-// eight waves, two row tiles each, one block a compute unit, with three buffers of tiles and the loads two tiles
-// ahead (issued by inline assembly: the compiler, which counts the loads into each LDS array itself, otherwise waits
-// for all of them before the first read of a tile): the same time where all blocks have long key ranges (2,048 tokens
-// after 26,000: 882 against 888 us) and 4 to 25 % more for portions without earlier keys, whose one block a unit cannot
-// pair a long key range with a short one. So the kernel waits neither for its tiles to arrive nor for a better order
-// of its own instructions: its time is about that of its matrix instructions plus that of its vector instructions,
-// one after the other (per 64-key tile and wave 64 x 16 clocks and about 1,200, measured 2,550 for the two waves of a
-// SIMD together), as if the two kinds did not overlap; a microbenchmark of both kinds interleaved in one wave shows
-// half of the vector instructions' time hidden at best.
-// (When kernels are compared, the first one or two of a process run up to a tenth slower than later ones: what is
-// compared has to be run in turn, more than once.)
 #include "nhv_common.h"
 #include <math.h>
 #include <type_traits>

@@ -4,24 +4,30 @@
 #include "nhv_common.h"
 
 // ---------------------------------------------------------------- embedding
+// scale: the row is multiplied by it in float and rounded once (1: the row is copied as it is)
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, T* __restrict__ out,
-                             int H, int V) {
+                             int H, int V, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   const bool ok = id >= 0 && id < V;   // the host checks ids; an id out of range gives a row of zeros, never a wild read
   const T* src = table + (size_t)(ok ? id : 0) * H;
   T* dst = out + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ok ? src[i] : from_f32<T>(0.f);
+  if (scale == 1.0f) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ok ? src[i] : from_f32<T>(0.f);
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ok ? from_f32<T>(to_f32(src[i]) * scale) : from_f32<T>(0.f);
+  }
 }
 
-extern "C" int nhv_embed(const void* ids, const void* table, void* out, int T, int H, int V, int dtype, void* stream) {
+extern "C" int nhv_embed(const void* ids, const void* table, void* out, int T, int H, int V, int dtype, float scale,
+                         void* stream) {
   NHV_REQUIRE(T > 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == NHV_F32)
-    hipLaunchKernelGGL(embed_kernel<float>, dim3(T), dim3(256), 0, s, (const int*)ids, (const float*)table, (float*)out, H, V);
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(T), dim3(256), 0, s, (const int*)ids, (const float*)table, (float*)out, H, V, scale);
   else if (dtype == NHV_BF16)
-    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (const int*)ids, (const bf16_t*)table, (bf16_t*)out, H, V);
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (const int*)ids, (const bf16_t*)table, (bf16_t*)out, H, V, scale);
   else
     return nhv_fail("embed: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("embed");
@@ -259,6 +265,22 @@ extern "C" int nhv_gather_rows(const void* x, const void* rows, void* out, int n
   return 0;
 }
 
+// ---------------------------------------------------------------- a soft cap on float logits, in place
+__global__ void soft_cap_kernel(float* __restrict__ x, size_t n, float cap) {
+  const float inv = 1.0f / cap;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    x[i] = cap * tanhf(x[i] * inv);
+}
+
+extern "C" int nhv_soft_cap(void* x, size_t n, float cap, void* stream) {
+  NHV_REQUIRE(n > 0 && cap > 0.f, "soft_cap: needs entries and a positive cap (n=%zu, cap=%g)", n, (double)cap);
+  const size_t want = (n + 255) / 256;
+  hipLaunchKernelGGL(soft_cap_kernel, dim3((unsigned)(want > 65535 * 8 ? 65535 * 8 : want)), dim3(256), 0, (hipStream_t)stream,
+                     (float*)x, n, cap);
+  NHV_LAUNCH_CHECK("soft_cap");
+  return 0;
+}
+
 // ---------------------------------------------------------------- q/k norm + rotation + cache write
 // One wave per (token, head) of the packed projection qkv[T, (Hq + 2 Hkv) D]
 // (+ bias). q and k heads: optional RMSNorm over the head (rounded, then times
@@ -266,11 +288,14 @@ extern "C" int nhv_gather_rows(const void* x, const void* rows, void* out, int n
 // (j, j + rot/2) by the angle of the token's position. q goes to q_out[T, Hq, D];
 // k and v go into the paged cache at slot_mapping[t] (a negative slot is skipped).
 // cos_sin: [max_pos, rot] float, cos in the first rot/2 columns, sin in the rest.
+// positions: [axes, T]; pair_axes (may be null: every pair turns by axis 0): [rot/2], the axis whose coordinate
+// gives pair j its angle (the table's row is then looked up pair by pair).
 template <typename T, typename W>
 __global__ void qk_rope_write_kernel(const T* __restrict__ qkv, const T* __restrict__ bias,
                                      const W* __restrict__ q_norm_w, const W* __restrict__ k_norm_w, float eps,
                                      const float* __restrict__ cos_sin, int rot,
-                                     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
+                                     const int* __restrict__ positions, const int* __restrict__ pair_axes, int n_tokens,
+                                     const int* __restrict__ slot_mapping,
                                      T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                      int Hq, int Hkv, int D, int heads_per_token) {
   extern __shared__ float head[];          // D floats
@@ -314,14 +339,13 @@ __global__ void qk_rope_write_kernel(const T* __restrict__ qkv, const T* __restr
   __syncthreads();                          // one wave per block: orders the LDS writes before the paired reads
   T* dst = is_q ? q_out + ((size_t)t * Hq + h) * D : k_cache + ((size_t)slot * Hkv + (h - Hq)) * D;
   const int half = rot / 2;
-  const float* cs = cos_sin + (size_t)positions[t] * rot;
   for (int d = lane; d < D; d += NHV_WAVE) {
     float out;
-    if (d < half) {
-      out = head[d] * cs[d] - head[d + half] * cs[half + d];
-    } else if (d < rot) {
-      const int j = d - half;
-      out = head[d] * cs[j] + head[j] * cs[half + j];
+    if (d < rot) {
+      const int j = d < half ? d : d - half;
+      const int axis = pair_axes ? pair_axes[j] : 0;
+      const float* cs = cos_sin + (size_t)positions[(size_t)axis * n_tokens + t] * rot;
+      out = d < half ? head[d] * cs[j] - head[d + half] * cs[half + j] : head[d] * cs[j] + head[j] * cs[half + j];
     } else {
       out = head[d];
     }
@@ -400,7 +424,7 @@ __global__ __launch_bounds__(256) void qk_rope_write_vec_kernel(
 }
 
 extern "C" int nhv_qk_rope_write(const void* qkv, const void* bias, const void* q_norm_w, const void* k_norm_w, float eps,
-                                 const void* cos_sin, int rot, int max_pos, const void* positions,
+                                 const void* cos_sin, int rot, int max_pos, const void* positions, const void* pair_axes,
                                  const void* slot_mapping, void* q_out, void* k_cache, void* v_cache, int T, int Hq,
                                  int Hkv, int D, int write_kv, int dtype, int w_dtype, void* stream) {
   NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && D > 0, "qk_rope_write: bad sizes T=%d Hq=%d Hkv=%d D=%d", T, Hq, Hkv, D);
@@ -418,7 +442,7 @@ extern "C" int nhv_qk_rope_write(const void* qkv, const void* bias, const void* 
   const bool aligned = (uintptr_t)qkv % 16 == 0 && (uintptr_t)q_out % 16 == 0 && (uintptr_t)k_cache % 16 == 0 &&
                        (uintptr_t)v_cache % 16 == 0 && (uintptr_t)bias % 16 == 0 && (uintptr_t)q_norm_w % 16 == 0 &&
                        (uintptr_t)k_norm_w % 16 == 0 && (uintptr_t)cos_sin % 16 == 0;
-  if (pow2 && aligned && (rot == D || rot == 0)) {
+  if (pow2 && aligned && (rot == D || rot == 0) && pair_axes == nullptr) {
     const long long n_items = (long long)T * heads;
     const long long vblocks = (n_items * ch + 255) / 256;
     NHV_REQUIRE(vblocks <= 0x7fffffff, "qk_rope_write: too many tokens");
@@ -448,8 +472,8 @@ extern "C" int nhv_qk_rope_write(const void* qkv, const void* bias, const void* 
 #define LAUNCH(TT, WW)                                                                                              \
   hipLaunchKernelGGL((qk_rope_write_kernel<TT, WW>), dim3((unsigned)((size_t)T * heads)), dim3(NHV_WAVE), lds, s,  \
                      (const TT*)qkv, (const TT*)bias, (const WW*)q_norm_w, (const WW*)k_norm_w, eps,               \
-                     (const float*)cos_sin, rot, (const int*)positions, (const int*)slot_mapping, (TT*)q_out,       \
-                     (TT*)k_cache, (TT*)v_cache, Hq, Hkv, D, heads)
+                     (const float*)cos_sin, rot, (const int*)positions, (const int*)pair_axes, T,                  \
+                     (const int*)slot_mapping, (TT*)q_out, (TT*)k_cache, (TT*)v_cache, Hq, Hkv, D, heads)
   if (dtype == NHV_F32 && w_dtype == NHV_F32) LAUNCH(float, float);
   else if (dtype == NHV_BF16 && w_dtype == NHV_BF16) LAUNCH(bf16_t, bf16_t);
   else if (dtype == NHV_BF16 && w_dtype == NHV_F32) LAUNCH(bf16_t, float);

@@ -128,13 +128,7 @@ typedef const __attribute__((address_space(1))) void* global_ptr;
 // LDS buffers (one barrier a tile), and the waves take turns in adding them up and writing the result.
 // The first weights of a block's first tile are asked for right after x and the wait before the first product is for
 // x alone (0.2 to 0.5 us less per call at every shape; asked for before x they made every shape slower, by 0.5 to
-// 3 us). (Asking for the next tile's first loads before a tile's sums are exchanged was measured and changed nothing.
-// So was a walk in which a block's tiles turn over the XCDs from round to round: within 2 % either way, except the
-// 151,936-row head at 8 and 16 rows, 4 to 6 % less. And a range of rows of the same length for every block, taken 16 at
-// a time, instead of whole tiles dealt out in turn, so that every compute unit reads the same number of bytes (6,144
-// rows are 384 tiles, one and a half per unit): 5 to 8 % less time for some shapes at 8 rows, 5 to 35 % more for
-// others and at 1 row, with 256, 512 and 768 blocks alike; what the waves of a unit keep in flight counts for more
-// than the balance. Grids that are no multiple of the 256 units are 10 to 40 % slower.)
+// 3 us).
 template <int WAVES, int UNROLL, bool GLU, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                            const bf16_t* __restrict__ bias, TOut* __restrict__ y,

@@ -16,7 +16,13 @@
 //  * All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads)
 //    race. The array keeps the last call's contents; nothing in it has to start at zero, since a call reads
 //    only the entries that it has written itself.
-//  * Arguments are those of nhv_decode_attention_bf16, in its order, without part_o and part_ml.
+//  * Arguments are those of nhv_decode_attention_bf16, in its order, without part_o and part_ml. As there,
+//    n_splits * split_len must cover every position of the batch: a token whose position lies beyond loses the
+//    keys of the splits that were not launched (nothing is read past the array).
+//  * The first call on a device asks the runtime for the array's address on that device (a symbol lookup, under
+//    a lock). That one call must not happen while a stream of the device is being captured into a graph: call
+//    nhv_decode_attention_no_alloc_init() (which allocates nothing either) or make one ordinary call on every
+//    device first; later calls only launch kernels and may be recorded.
 #pragma once
 #include <stddef.h>
 
@@ -27,6 +33,10 @@ extern "C" int nhv_decode_attention_bf16_no_alloc(const void* q, const void* k_c
                                                   const void* block_tables, int max_blocks, int T, int Hq, int Hkv,
                                                   int page_size, float scale, int window, int split_len, int n_splits,
                                                   void* stream);
+
+// asks for the array's address on the current device and keeps it (0, or 1 with nhv_last_error() set); a
+// call on a device whose address is known already does nothing
+extern "C" int nhv_decode_attention_no_alloc_init();
 
 // bytes of the scratch array (NHV_NO_ALLOC_SCRATCH_BYTES), for callers that size their calls by it
 extern "C" size_t nhv_decode_attention_no_alloc_limit();

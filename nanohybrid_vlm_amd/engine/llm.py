@@ -94,13 +94,35 @@ def _load_tokenizer(folder: str):
     return Tokenizer.from_file(path)
 
 
+def _tokenizer_eos(folder: str, tokenizer) -> int | None:
+    """The id of the tokenizer's end-of-sequence token: ``tokenizer_config.json`` names the token (a string, or an
+    object with ``content``), ``tokenizer.json`` knows its id. None if the folder does not say. Several end tokens
+    are refused, as for the model's own (nanovllm/engine/llm_engine.py:217-220)."""
+    import json
+    path = os.path.join(folder, "tokenizer_config.json")
+    if tokenizer is None or not os.path.isfile(path):
+        return None
+    with open(path) as f:
+        token = json.load(f).get("eos_token")
+    if isinstance(token, dict):
+        token = token.get("content")
+    if isinstance(token, (list, tuple)):
+        raise NotImplementedError("several end-of-sequence tokens are not supported")
+    if not isinstance(token, str):
+        return None
+    return tokenizer.token_to_id(token)
+
+
 class LLM:
-    def __init__(self, model, *, random_weights: int | None = None, built_model=None, **kwargs):
+    def __init__(self, model, *, random_weights: int | None = None, built_model=None, poison_freed_pages: bool = False,
+                 **kwargs):
         """``model``: folder with config.json, model.safetensors (and tokenizer.json for text prompts); or the
         contents of a config.json as a dict, together with ``random_weights=seed``: a model of that
         configuration with random weights drawn on the device.
         ``built_model``: (architecture, typed configuration, model with weights bound) made elsewhere;
-        ``model`` is then only a label."""
+        ``model`` is then only a label.
+        ``poison_freed_pages``: a debugging aid of the runner (every page that a request gives back is filled
+        with NaN, so that a read of a page its reader no longer owns shows in the logits)."""
         unknown = set(kwargs) - EngineConfig.field_names()
         if unknown:
             raise TypeError(f"unknown engine options: {sorted(unknown)}; known: {sorted(EngineConfig.field_names())}")
@@ -111,7 +133,8 @@ class LLM:
                 raise TypeError("a configuration in place of a model folder needs random_weights=SEED")
             from ..weights.random_init import build_random_model
             check = EngineConfig(model="random weights", **kwargs)           # (the options are checked before the weights are drawn)
-            built_model = build_random_model(model, random_weights, check.dtype, check.device)
+            built_model = build_random_model(model, random_weights, check.dtype, check.device,
+                                             options={"residual_float32": check.residual_dtype == "float32"})
             model = f"random weights ({built_model[0].name}, seed {random_weights})"
         elif random_weights is not None:
             raise TypeError("random_weights goes with a configuration (a dict), not with a model folder")
@@ -127,16 +150,23 @@ class LLM:
             gpu_memory_utilization=cfg.gpu_memory_utilization, max_num_batched_tokens=cfg.max_num_batched_tokens,
             model=built, arch=arch, cfg=typed, use_graphs=not cfg.enforce_eager, max_model_len=cfg.max_model_len,
             share_prefixes=cfg.enable_prefix_cache, max_graph_batch=cfg.max_graph_batch, max_graph_tokens=cfg.max_graph_tokens,
-            residual_float32=cfg.residual_dtype == "float32")
+            residual_float32=cfg.residual_dtype == "float32", poison_freed_pages=poison_freed_pages)
         cfg.num_kvcache_blocks = self.runner.num_pages
         # max_model_len is capped by the model's positions (nanovllm/config.py:420-423); both, and the token that
         # ends a request, are facts of the built model (no field of an architecture's configuration is read here)
         cfg.max_model_len = min(cfg.max_model_len, self.runner.max_position)
-        if cfg.eos == -1 and self.runner.eos_token_id is not None:
-            cfg.eos = self.runner.eos_token_id
         self.tokenizer = _load_tokenizer(model) if built_model is None else None
+        if cfg.eos == -1:
+            # the model's end token; a model that names none ends where its tokenizer does
+            # (nanovllm/engine/llm_engine.py:207-223)
+            eos = self.runner.eos_token_id
+            if eos is None and built_model is None:
+                eos = _tokenizer_eos(model, self.tokenizer)
+            if eos is not None:
+                cfg.eos = eos
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.eos,
-                                   cfg.max_model_len, cfg.scheduler_policy, cfg.max_prefill_wait_ms)
+                                   cfg.max_model_len, cfg.scheduler_policy, cfg.max_prefill_wait_ms,
+                                   release=self.runner.finish)
         self.sampler = Sampler(self.runner.vocab_size)
         self._ids = count()
         self._sequences: dict[int, Sequence] = {}
@@ -205,7 +235,7 @@ class LLM:
         counts = token_counts if token_counts is not None else runner.mixed_token_buckets
         for t in counts:
             if t <= min(runner.max_graph_tokens, runner.max_model_len, runner.num_pages * runner.page_size):
-                runner.step([StepEntry(("warm up", 0), [0] * t, [t - 1])])
+                runner.step([StepEntry(("warm up", 0), [0] * (t - 1), [t - 2])])   # (a bucket holds steps of fewer tokens than its size)
                 runner.finish(("warm up", 0))
         stats = runner.get_memory_stats()
         return {key: stats[key] for key in ("graphs_recorded", "mixed_graphs_recorded")}

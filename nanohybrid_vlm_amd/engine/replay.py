@@ -8,7 +8,9 @@ A step is a dict, one line of JSON in a trace file:
 
 ``entries``: for each request its next tokens and the places among them whose logits
 are wanted; all entries of a step are one batch. ``end``: requests that are over
-after this step; what they hold in the cache is given back.
+after this step; what they hold in the cache is given back. An entry may also bring
+``"positions": [[...], ...]``, its tokens' positions as the position encodings see
+them, one list per position axis of the model (default: the tokens' indices).
 
 A whole trace may also come as one JSON object that names the requests' tokens once and
 then says, step by step, how many of its next tokens each request feeds:
@@ -58,7 +60,8 @@ def make_runner(model_dir: str, dtype: str, max_tokens: int, page_size: int = 64
 def replay_step(runner: ModelRunner, record: dict) -> torch.Tensor | None:
     """Runs one step of a trace. Returns float32 logits [wanted, vocab] in the order of the entries and of each
     entry's ``want``, or None if the step wants nothing (or brings nothing)."""
-    entries = [StepEntry(e["id"], list(e["tokens"]), list(e.get("want") or [])) for e in record.get("entries") or []]
+    entries = [StepEntry(e["id"], list(e["tokens"]), list(e.get("want") or []), e.get("positions"))
+               for e in record.get("entries") or []]
     logits = runner.step(entries) if entries else None
     for request_id in record.get("end") or []:
         runner.finish(request_id)

@@ -41,6 +41,10 @@ class StepEntry:
     request_id: Hashable
     tokens: list[int]                       # its next tokens (at least one)
     want: list[int] = field(default_factory=list)   # places among ``tokens`` whose logits are returned
+    # the tokens' positions as the position encodings see them, [axes][tokens]; None: on every axis a token's
+    # position is its index in the request. (Where a token's key is stored and which keys it may read follows
+    # from its index alone.)
+    positions: list[list[int]] | None = None
 
 
 class ModelRunner:
@@ -59,26 +63,24 @@ class ModelRunner:
             raw = read_config_json(model_dir)
             arch = resolve_architecture(raw)
             cfg = arch.parse_config(raw)
-            model = DecoderModel(arch.build_spec(cfg))
+            # engine options that parts may care for are offered to every part's constructor
+            model = DecoderModel(arch.build_spec(cfg), options={"residual_float32": bool(residual_float32)})
             load_weights(model, arch, cfg, model_dir, self.dtype, self.device)
         self.arch, self.cfg, self.model = arch, cfg, model
         self.model.to(self.device)
-        # an engine option that parts carry as an attribute: whether the residual stream keeps float32 between layers
-        for part in self.model.walk():
-            if hasattr(part, "residual_float32"):
-                part.residual_float32 = bool(residual_float32)
         # what the engine above needs to know of the model comes from the model's description, not from the
         # architecture's typed configuration (whose fields are the architecture's own affair)
         self.vocab_size = model.spec.vocab_size
         self.max_position = model.spec.max_position
         self.eos_token_id = model.spec.eos_token_id
         self.page_size = page_size
+        # a model whose positions have several coordinates gets them as an array of their own in every step; for the
+        # others the tokens' indices are the positions, unless an entry brings positions of its own
+        self.position_axes = model.spec.position_axes
         if share_prefixes and poison_freed_pages:
             raise ValueError("a freed page keeps its content for later requests when prefixes are shared; "
                              "poison_freed_pages would destroy it")
         self.share_prefixes = share_prefixes
-        self._make_cache(page_size, num_pages, num_state_slots, gpu_memory_utilization, max_num_batched_tokens,
-                         graph_rows=max_graph_batch if use_graphs else 0, graph_tokens=max_graph_tokens if use_graphs else 0)
         self._pinned = None
         self._pinned_free = None
         # a debugging aid: pages that are given back are filled with NaN, so that a read of a page that a
@@ -109,44 +111,58 @@ class ModelRunner:
         self._mixed_graphs: dict[tuple[int, int], dict | None] = {}
         self.graph_check = torch.equal                # (replay, eager) -> bool; a test replaces it to force a refusal
         self.graphs_rerecorded = 0                    # graphs recorded again because the contexts had outgrown their layout
+        # all recorded steps share one pool of memory: they replay one after the other on one stream, so what one
+        # needs between its kernels can be what another needed; each keeps only its own logits and index arrays
+        self._graph_pool = None
+        self.probe = None                             # what the cache's sizing measured (see _pages_from_free_memory)
+        self._make_cache(page_size, num_pages, num_state_slots, gpu_memory_utilization, max_num_batched_tokens)
 
     # ------------------------------------------------------------------ cache
-    def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens, graph_rows=0, graph_tokens=0):
+    def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens):
         needs = self.model.cache_needs()
         windows: list[int | None] = []                 # one group per distinct window
-        entry_group: dict[int, int] = {}
+        self._entry_group: dict[int, int] = {}
         for i, need in enumerate(needs):
             if isinstance(need, PagedKVNeed):
                 if need.window not in windows:
                     windows.append(need.window)
-                entry_group[i] = windows.index(need.window)
+                self._entry_group[i] = windows.index(need.window)
         if not windows:
             windows = [None]                           # a model without paged layers still has one (empty) group
+        self._windows = windows
         if self.share_prefixes and any(isinstance(n, StateNeed) for n in needs):
             # state of fixed size summarises all earlier tokens: pages alone do not bring a prefix back
             # (the reference switches the page hashes off for such models, nanovllm/config.py:384-399)
             raise ValueError("prefixes cannot be shared by a model with per-request state")
-        views: list[CacheView | None] = [None] * len(needs)
         # the pools of per-request state come first, so that the pages are counted from what is left
         # (the reference splits its budget between the two, nanovllm/engine/model_runner.py:723-775).
         # One row more than there are slots: the padding rows of a recorded step work on it.
         self.state_pools: list[dict] = []
+        self._state_views: dict[int, CacheView] = {}
         self.num_state_slots = num_state_slots
         for i, need in enumerate(needs):
             if isinstance(need, StateNeed):
                 pool = {name: torch.zeros((num_state_slots + 1, *shape), dtype=dt, device=self.device)
                         for name, (shape, dt) in need.tensors.items()}
                 self.state_pools.append(pool)
-                views[i] = CacheView(kind="state", state=pool)
+                self._state_views[i] = CacheView(kind="state", state=pool)
         item = torch.empty((), dtype=self.dtype).element_size()
         page_bytes = sum(2 * page_size * n.num_kv_heads * n.head_dim * item
                          for n in needs if isinstance(n, PagedKVNeed))
         if num_pages is None:
-            num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens, graph_rows, graph_tokens)
+            num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens)
+        self._allocate_pages(num_pages)
+
+    def _allocate_pages(self, num_pages: int) -> None:
+        """The cache manager and the key/value tensors for ``num_pages`` pages per group, attached to the model."""
+        needs = self.model.cache_needs()
+        page_size = self.page_size
         self.num_pages = num_pages
         groups = [PagedGroupSpec(name="all keys" if w is None else f"window {w}", page_size=page_size,
-                                 num_pages=num_pages, window=w) for w in windows]
-        self.cache = CacheManager(groups, num_state_slots, share_prefixes=self.share_prefixes)
+                                 num_pages=num_pages, window=w) for w in self._windows]
+        self.cache = CacheManager(groups, self.num_state_slots, share_prefixes=self.share_prefixes)
+        views: list[CacheView | None] = [None] * len(needs)
+        views[:] = [self._state_views.get(i) for i in range(len(needs))]
         self.kv_tensors: list[torch.Tensor] = []       # the pages that requests may hold, per cache unit
         for i, need in enumerate(needs):
             if isinstance(need, PagedKVNeed):
@@ -157,7 +173,7 @@ class ModelRunner:
                                  dtype=self.dtype, device=self.device)
                 kv[:, num_pages].zero_()
                 self.kv_tensors.append(kv[:, :num_pages])
-                views[i] = CacheView(kind="paged", group=entry_group[i], k=kv[0], v=kv[1], writes=True)
+                views[i] = CacheView(kind="paged", group=self._entry_group[i], k=kv[0], v=kv[1], writes=True)
         for i, e in enumerate(self.model.run_order):
             if e.cache is not None:
                 lender = views[e.cache]
@@ -167,31 +183,98 @@ class ModelRunner:
                 views[i] = CacheView(kind="none")
         self.model.attach_cache(views)
 
-    def _pages_from_free_memory(self, page_bytes, utilization, max_tokens, graph_rows, graph_tokens=0) -> int:
+    def _pages_from_free_memory(self, page_bytes, utilization, max_tokens) -> int:
         """budget = total * utilization - used - room for a step's activations - room for the recorded steps
-        (nanovllm/engine/model_runner.py:654-699,839-861; the reference measures the room with a warm-up pass,
-        here it is computed from the layer sizes). The weights and the state pools are allocated already and
-        count as used."""
+        (nanovllm/engine/model_runner.py:654-699,839-861). As the reference does, the room is measured, not
+        computed: on a cache just large enough for it, the largest step that the engine can be asked for is run
+        once eagerly (``max_tokens`` tokens of as many requests as there are state slots, every request wanting
+        a row of logits) and the allocator's peak over what it held before is the activations' room; the
+        largest recorded steps of both kinds are recorded once, and what they add to the allocator's reserve
+        beyond their own logits is the room of the pool that all recorded steps share. Every recorded step's own
+        logits and index arrays are counted by their sizes. Then the probe's cache is given back and the pages
+        are what the budget has left. The weights and the state pools are allocated already and count as used."""
         if page_bytes == 0:
             return 1
         free, total = torch.cuda.mem_get_info(self.device)
-        s = self.model.spec
-        widest = 0
-        for name, spec in self.model.all_param_specs().items():
-            if len(spec.shape) == 2 and not name.startswith(("embed.", "head.")):
-                widest = max(widest, spec.shape[0])
-        item = torch.empty((), dtype=self.dtype).element_size()
-        activations = max_tokens * (3 * widest + 8 * s.hidden_size) * item + 2 * 512 * s.vocab_size * 4
-        # every recorded batch size keeps its own logits and a step's activations of that many rows
-        buckets = [b for b in self._bucket_sizes(graph_rows)] if graph_rows else []
-        recorded = sum(b * (s.vocab_size * 4 + (3 * widest + 8 * s.hidden_size) * item) + (64 << 20) for b in buckets)
-        # and every recorded short step of any make: its tokens' activations and its requests' logits
-        if graph_rows and graph_tokens:
-            for t in self._token_bucket_sizes(graph_tokens):
-                for b in [b for b in (1, 4, 16, 64) if b < graph_rows] + [graph_rows]:
-                    recorded += t * (3 * widest + 8 * s.hidden_size) * item + b * s.vocab_size * 4 + (32 << 20)
-        budget = total * utilization - (total - free) - activations - recorded
+        # the probe's step: single tokens of all but one request, the rest of the tokens in requests as long as allowed
+        tokens = max(1, max_tokens)
+        slots = max(1, self.num_state_slots)
+        lengths = [1] * min(slots - 1, max(0, tokens - 1))
+        rest = tokens - len(lengths)
+        while rest > 0 and len(lengths) < slots:
+            n = min(rest, self.max_model_len)
+            lengths.append(n)
+            rest -= n
+        probe_pages = sum(-(-n // self.page_size) for n in lengths)
+        if (probe_pages + 1) * page_bytes > total * utilization - (total - free):
+            raise RuntimeError(f"no memory left for the cache: {free / 2**30:.1f} GiB free of {total / 2**30:.1f}; the "
+                               f"largest step alone needs {probe_pages} pages of {page_bytes / 2**20:.1f} MiB")
+        self._allocate_pages(probe_pages)
+        try:
+            torch.cuda.synchronize(self.device)
+            torch.cuda.reset_peak_memory_stats(self.device)
+            held = torch.cuda.memory_allocated(self.device), torch.cuda.memory_reserved(self.device)
+            entries = [StepEntry(("probe", i), [0] * n, [n - 1]) for i, n in enumerate(lengths)]
+            logits = self.step(entries)
+            torch.cuda.synchronize(self.device)
+            del logits
+            activations = max(torch.cuda.max_memory_allocated(self.device) - held[0],
+                              torch.cuda.max_memory_reserved(self.device) - held[1])
+            for e in entries:
+                self.finish(e.request_id)
+            shared_pool, own = 0, 0
+            s = self.model.spec
+            if self.use_graphs:
+                width = -(-self.max_model_len // self.page_size)
+                # the largest recorded step of single tokens and the largest of any other make, recorded here once
+                most = min(self.max_graph_batch, slots, probe_pages)
+                bucket = max([b for b in self.graph_buckets if b <= most], default=None)
+                def reserved() -> int:                 # what the allocator holds, without blocks it only keeps for later
+                    torch.cuda.synchronize(self.device)
+                    torch.cuda.empty_cache()
+                    return torch.cuda.memory_reserved(self.device)
+
+                if bucket is not None:
+                    before = reserved()
+                    ids = [("probe", i) for i in range(bucket)]
+                    self.step([StepEntry(r, [0], []) for r in ids])
+                    self.step([StepEntry(r, [0], [0]) for r in ids])
+                    for r in ids:
+                        self.finish(r)
+                    shared_pool += max(0, reserved() - before - bucket * s.vocab_size * 4)
+                t = max([t for t in self.mixed_token_buckets if t - 1 <= min(self.max_model_len, probe_pages * self.page_size)],
+                        default=None)
+                if t is not None and t >= 2:
+                    before = reserved()
+                    self.step([StepEntry(("probe", 0), [0] * (t - 1), [t - 2])])
+                    self.finish(("probe", 0))
+                    shared_pool += max(0, reserved() - before - s.vocab_size * 4)
+                # every recorded step's own: float32 logits of its rows, and its index arrays (block tables of full width)
+                row = s.vocab_size * 4 + (width * len(self._windows) + 16) * 4
+                own = sum(b * row for b in self.graph_buckets)
+                own += sum(rb * row + tb * 16 for tb in self.mixed_token_buckets for rb in self.mixed_request_buckets)
+                # and the matrix products of every new size of step are timed once: a sweep of the caches and a workspace
+                from ..native import ops
+                backend = ops.backend()
+                if getattr(backend, "measuring_allowed", False):
+                    own += (512 << 20) + 2 * getattr(backend, "library_workspace", 0)
+        finally:
+            # the probe's cache, its graphs and whatever the allocator kept go back to the device
+            self._graphs.clear()
+            self._mixed_graphs.clear()
+            self._graph_pool = None
+            self.graphs_rerecorded = 0
+            self.model.attach_cache([CacheView(kind="none") for _ in self.model.run_order])
+            self.kv_tensors = []
+            self.cache = None
+            self._pinned = self._pinned_free = None
+            torch.cuda.synchronize(self.device)
+            torch.cuda.empty_cache()
+        free, total = torch.cuda.mem_get_info(self.device)
+        budget = total * utilization - (total - free) - activations - shared_pool - own
         pages = int(budget // page_bytes)
+        self.probe = {"tokens": tokens, "requests": len(lengths), "activation_bytes": int(activations),
+                      "graph_pool_bytes": int(shared_pool), "graph_own_bytes": int(own)}
         if pages <= 0:
             raise RuntimeError(f"no memory left for the cache: {free / 2**30:.1f} GiB free of {total / 2**30:.1f}, "
                                f"one page needs {page_bytes / 2**20:.1f} MiB")
@@ -277,6 +360,14 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= w < n:
                     raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its {n} tokens")
+            if e.positions is not None:
+                if len(e.positions) != self.position_axes or any(len(row) != n for row in e.positions):
+                    raise ValueError(f"request {e.request_id!r}: positions must be [{self.position_axes}][{n}] "
+                                     f"(axes of the model, tokens of the entry)")
+                for row in e.positions:
+                    if min(row) < 0 or max(row) >= self.max_position:
+                        raise ValueError(f"request {e.request_id!r}: a position is outside the model's "
+                                         f"{self.max_position} positions")
             known = e.request_id in cache
             new_requests += not known
             new_len = (cache.num_tokens(e.request_id) if known else 0) + n
@@ -359,10 +450,24 @@ class ModelRunner:
                     raise RuntimeError(f"request {entries[i].request_id!r}: a new token falls on a page that was given back")
                 slot_mapping[cu[i]:cu[i + 1]] = pages * g.page_size + p % g.page_size
             arrays += [slot_mapping, bt]
+        arrays += self._position_rows(entries, positions, cu)
         meta = {"B": B + pad, "T": T, "rows": rows, "starts": starts, "new_lens": new_lens,
                 "q_lens": q_lens.tolist(), "state_slots": state_slots.tolist(),
                 "max_q_len": int(q_lens.max()), "max_context_len": int(max(new_lens))}
         return arrays, meta
+
+    def _position_rows(self, entries: list[StepEntry], index: np.ndarray, cu) -> list[np.ndarray]:
+        """The positions as the position encodings see them, [axes, T], as one more array of the step; nothing for a
+        model of one axis whose entries bring no positions of their own (the tokens' indices are the positions).
+        Padding tokens keep their index."""
+        explicit = any(e.positions is not None for e in entries)
+        if self.position_axes == 1 and not explicit:
+            return []
+        rows = np.repeat(index[None, :], self.position_axes, axis=0)
+        for i, e in enumerate(entries):
+            if e.positions is not None:
+                rows[:, int(cu[i]):int(cu[i + 1])] = np.asarray(e.positions, dtype=np.int32)
+        return [np.ascontiguousarray(rows, dtype=np.int32)]
 
     def _layout_single_tokens(self, entries: list[StepEntry], pad_to: int | None, table_width: int | None):
         """``_layout`` for a step in which every request brings one token (a decoding step): the same arrays,
@@ -403,6 +508,7 @@ class ModelRunner:
             flat += ([self.num_pages] + [NO_PAGE] * (width - 1)) * pad
             bt = np.array(flat, dtype=np.int32).reshape(n, width)
             arrays += [np.array(slot_mapping, dtype=np.int32), bt]
+        arrays += self._position_rows(entries, arrays[1], arrays[3])
         meta = {"B": n, "T": n, "rows": rows, "starts": starts, "new_lens": new_lens, "q_lens": [1] * n,
                 "state_slots": slots + [self.num_state_slots] * pad, "max_q_len": 1, "max_context_len": max(new_lens)}
         return arrays, meta
@@ -410,13 +516,15 @@ class ModelRunner:
     def _context(self, dev: list[torch.Tensor], meta: dict, logit_rows: torch.Tensor | None, num_logit_rows: int,
                  max_context_len: int) -> StepContext:
         d_ids, d_pos, d_req, d_cu, d_ctx, d_slots = dev[:6]
-        groups = [GroupTables(slot_mapping=dev[6 + 2 * gi], block_tables=dev[7 + 2 * gi])
-                  for gi in range(len(self.cache.groups))]
+        num_groups = len(self.cache.groups)
+        groups = [GroupTables(slot_mapping=dev[6 + 2 * gi], block_tables=dev[7 + 2 * gi]) for gi in range(num_groups)]
+        # the positions of the position encodings: an array of their own if the step carries one, else the indices
+        positions = dev[6 + 2 * num_groups] if len(dev) > 6 + 2 * num_groups else d_pos.view(1, -1)
         attention = AttentionBatch(num_tokens=meta["T"], num_requests=meta["B"], token_req=d_req, positions=d_pos,
                                    cu_seqlens_q=d_cu, context_lens=d_ctx, max_q_len=meta["max_q_len"],
                                    max_context_len=max_context_len)
-        return StepContext(num_tokens=meta["T"], num_requests=meta["B"], input_ids=d_ids, positions=d_pos,
-                           attention=attention, groups=groups, state_slots=d_slots, logit_rows=logit_rows,
+        return StepContext(num_tokens=meta["T"], num_requests=meta["B"], input_ids=d_ids, positions=positions,
+                           token_positions=positions[0], attention=attention, groups=groups, state_slots=d_slots, logit_rows=logit_rows,
                            num_logit_rows=num_logit_rows,
                            host={k: meta[k] for k in ("starts", "new_lens", "q_lens", "state_slots")})
 
@@ -434,15 +542,20 @@ class ModelRunner:
         """Runs the batch and returns float32 logits [wanted, vocab] in the order of the
         entries and of each entry's ``want`` (None if nothing is wanted). With ``keep=False`` the result may be
         memory that the next step overwrites (a caller that samples at once saves the copy)."""
-        if self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries):
+        # (a recorded step of a model with one position axis has no array for positions of an entry's own)
+        recorded = self.use_graphs and (self.position_axes > 1 or all(e.positions is None for e in entries))
+        if recorded and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries):
             bucket = next(b for b in self.graph_buckets if b >= len(entries))
             if self._graphs.get(bucket, ...) is not None:
                 return self._graph_step(entries, bucket, keep)
-        elif self.max_graph_tokens and len(entries) <= self.max_graph_batch and all(len(e.want) <= 1 for e in entries):
+        elif recorded and self.max_graph_tokens and len(entries) <= self.max_graph_batch and all(len(e.want) <= 1 for e in entries):
             tokens = sum(len(e.tokens) for e in entries)
-            if tokens <= self.max_graph_tokens:
-                key = (next(t for t in self.mixed_token_buckets if t >= tokens),
-                       next(b for b in self.mixed_request_buckets if b >= len(entries)))
+            # the bucket is strictly larger than the step: the request that owns the filling tokens has at least one,
+            # so every request of the padded batch, also one without tokens, has its first row inside the batch
+            # (a part may index rows by ``cu_seqlens_q[:-1]``)
+            token_bucket = next((t for t in self.mixed_token_buckets if t > tokens), None)
+            if token_bucket is not None:
+                key = (token_bucket, next(b for b in self.mixed_request_buckets if b >= len(entries)))
                 # (the tokens that fill a bucket stand at positions below the bucket's size: the model must have them)
                 if key[0] <= self.max_model_len and self._mixed_graphs.get(key, ...) is not None:
                     return self._mixed_graph_step(entries, key, keep)
@@ -477,11 +590,11 @@ class ModelRunner:
         # longest context is half as long again, or less than half of it, a new graph is recorded (the old one is dropped)
         # (no graph is made for less than 256 keys: short contexts share one)
         longest = max(256, meta["max_context_len"])
-        if g is None or not g["planned"] // 2 < longest <= g["planned"] + g["planned"] // 2:
+        if g is None or not g["planned"] // 2 < longest <= g["covered"]:
             self.graphs_rerecorded += g is not None
             # (a graph recorded again holds the same library calls as the one before it, which passed its check:
-            # it is not checked again, and a step that records again takes 4 step times instead of 10)
-            g = self._capture(bucket, arrays, meta, width, len(entries), check=g is None)
+            # it is replayed and compared once, not three times with eager work between)
+            g = self._capture(bucket, arrays, meta, width, len(entries), checks=3 if g is None else 1)
             self._graphs[bucket] = g if g["graph"] is not None else None
         if g["graph"] is not None:
             g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
@@ -509,7 +622,8 @@ class ModelRunner:
         arrays.append(np.array(rows + [0] * (request_bucket - len(rows)), dtype=np.int32))
         g = self._mixed_graphs.get(key)
         if g is None:
-            g = self._capture_mixed(key, arrays, meta, width, len(rows))
+            # (a step that wants no logits still has its first token's row computed by the graph: that row is compared)
+            g = self._capture_mixed(key, arrays, meta, width, max(len(rows), 1))
             self._mixed_graphs[key] = g if g["graph"] is not None else None
         if g["graph"] is not None:
             g["index"].copy_(self._fill_host_buffer(arrays), non_blocking=True)
@@ -545,7 +659,7 @@ class ModelRunner:
         for r in request_ids:
             for gi, n in enumerate(self.cache.pages_needed(r, self.cache.num_tokens(r) + 1)):
                 need[gi] += n
-        return (g["planned"] // 2 < longest <= g["planned"] + g["planned"] // 2 and real <= self.max_model_len
+        return (g["planned"] // 2 < longest <= g["covered"] and real <= self.max_model_len
                 and real <= self.max_position and all(n <= self.cache.num_free_pages(gi) for gi, n in enumerate(need)))
 
     @torch.no_grad()
@@ -611,18 +725,20 @@ class ModelRunner:
             offset += n
         return index, dev
 
-    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int, num_real: int, check: bool = True) -> dict:
+    def _capture(self, bucket: int, arrays: list[np.ndarray], meta: dict, width: int, num_real: int, checks: int = 3) -> dict:
         """The graph of a step of single tokens for ``bucket`` requests."""
         index, dev = self._index_buffer(arrays)
         all_rows = torch.arange(bucket, dtype=torch.int32, device=self.device)
         ctx = self._context(dev, meta, all_rows, bucket, max_context_len=width * self.page_size)
-        # the graph's launches are fixed: kernels that split the keys plan for this step's longest context (replays
-        # with other lengths stay right: the block tables and the splits' results are made for max_model_len)
+        # the graph's launches are fixed: kernels that split the keys plan for this step's longest context, and their
+        # splits (and the splits' results) cover contexts of up to half as much again; the block tables are made for
+        # max_model_len. The graph serves contexts from half of ``planned`` to ``covered`` and is replaced beyond.
         planned = max(256, meta["max_context_len"])
-        graph, logits = self._record(ctx, f"{bucket} requests", num_real, planned, check)
-        return {"graph": graph, "index": index, "logits": logits, "ctx": ctx, "planned": planned}
+        covered = planned + planned // 2                   # (the kernels cut it down to what the block tables can hold)
+        graph, logits = self._record(ctx, f"{bucket} requests", num_real, planned, checks, covered)
+        return {"graph": graph, "index": index, "logits": logits, "ctx": ctx, "planned": planned, "covered": covered}
 
-    def _record(self, ctx: StepContext, what: str, num_real: int, planned: int, check: bool = True):
+    def _record(self, ctx: StepContext, what: str, num_real: int, planned: int, checks: int = 3, covered: int = 0):
         """Runs the step of ``ctx`` once eagerly on its fixed buffers (so that every kernel library is loaded
         and the allocator is warm), then records it, and checks the graph if a library call went into it. Returns
         (graph, its logits), or (None, the eager step's logits) if the step cannot be recorded or its graph fails.
@@ -632,10 +748,11 @@ class ModelRunner:
         backend = ops.backend()
         with_library = self.dtype == torch.bfloat16           # (the float32 path has kernels of its own throughout)
         old = (getattr(backend, "own_kernels_only", False), getattr(backend, "planned_context", 0),
-               getattr(backend, "measure_linears", False))
+               getattr(backend, "measure_linears", False), getattr(backend, "covered_context", 0))
         backend.own_kernels_only = False
         backend.measure_linears = True                        # few-rows products of new shapes are timed both ways, once
         backend.planned_context = planned
+        backend.covered_context = covered
         state_slots = ctx.state_slots.long()
         found = [{name: t[state_slots] for name, t in pool.items()} for pool in self.state_pools]
 
@@ -650,14 +767,16 @@ class ModelRunner:
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             try:
-                with torch.cuda.graph(graph):
+                if self._graph_pool is None:
+                    self._graph_pool = torch.cuda.graph_pool_handle()
+                with torch.cuda.graph(graph, pool=self._graph_pool):
                     logits = self.model.logits(self.model.forward(ctx))
             except RuntimeError as err:                       # something in the step cannot be recorded
                 print(f"[nanohybrid_vlm_amd] no graph for {what} ({str(err).splitlines()[0][:200]}); "
                       "steps of this size run eagerly", file=sys.stderr, flush=True)
                 return None, eager
-            if check and (with_library or self.state_pools):
-                for _ in range(3):
+            if with_library or self.state_pools:
+                for _ in range(checks):
                     logits.fill_(float("nan"))
                     put_state_back()
                     graph.replay()
@@ -667,12 +786,13 @@ class ModelRunner:
                         print(f"[nanohybrid_vlm_amd] the graph for {what} differs from the eager step when "
                               "replayed; steps of this size run eagerly", file=sys.stderr, flush=True)
                         return None, eager
-                    put_state_back()
-                    self.model.logits(self.model.forward(ctx))      # eager work between the replays
-                    torch.cuda.synchronize()
+                    if checks > 1:
+                        put_state_back()
+                        self.model.logits(self.model.forward(ctx))      # eager work between the replays
+                        torch.cuda.synchronize()
             put_state_back()                                  # the caller replays the graph for this very step
         finally:
-            backend.own_kernels_only, backend.planned_context, backend.measure_linears = old
+            backend.own_kernels_only, backend.planned_context, backend.measure_linears, backend.covered_context = old
             if hasattr(backend, "end_measurements"):
                 backend.end_measurements()
         return graph, logits
@@ -699,6 +819,7 @@ class ModelRunner:
             "graphs_recorded": sorted(b for b, g in self._graphs.items() if g is not None),
             "graphs_refused": sorted(b for b, g in self._graphs.items() if g is None),
             "graphs_rerecorded": self.graphs_rerecorded,
+            "cache_sizing_probe": self.probe,
             "mixed_graphs_recorded": sorted(k for k, g in self._mixed_graphs.items() if g is not None),
             "mixed_graphs_refused": sorted(k for k, g in self._mixed_graphs.items() if g is None),
         }

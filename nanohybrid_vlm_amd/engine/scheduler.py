@@ -80,7 +80,10 @@ class _Room:
 class Scheduler:
     def __init__(self, cache: CacheManager, max_num_seqs: int, max_num_batched_tokens: int, eos: int,
                  max_model_len: int, scheduler_policy: str = "decode_first", max_prefill_wait_ms: float = 50.0,
-                 clock: Callable[[], float] = monotonic):
+                 clock: Callable[[], float] = monotonic, release: Callable | None = None):
+        """``release``: how a request's pages and state slot are given back (default: the cache manager's own
+        ``release``); the engine passes the runner's ``finish``, so that whatever the runner does with pages that
+        come back (its ``poison_freed_pages``) also holds for requests that finish or are pushed out here."""
         if scheduler_policy not in ("decode_first", "prefill_first"):
             raise ValueError("scheduler_policy must be 'decode_first' or 'prefill_first'")
         self.cache = cache
@@ -91,6 +94,7 @@ class Scheduler:
         self.scheduler_policy = scheduler_policy
         self.max_prefill_wait_ms = max_prefill_wait_ms
         self.clock = clock
+        self.release = release if release is not None else cache.release
         self.waiting: deque[Sequence] = deque()       # arrival order; the head may hold pages already (a prompt under way)
         self.running: deque[Sequence] = deque()       # requests whose prompt is in the cache
         self.waiting_since: dict[int, float] = {}
@@ -235,7 +239,7 @@ class Scheduler:
         seq.num_cached_tokens = 0
         seq.num_scheduled_tokens = 0
         if seq.seq_id in self.cache:
-            self.cache.release(seq.seq_id)
+            self.release(seq.seq_id)
         self._enqueue(seq)
 
     # ------------------------------------------------------------------ after the step
@@ -254,7 +258,7 @@ class Scheduler:
             seq.append_token(token_id)
             if (not seq.ignore_eos and token_id == self.eos) or seq.num_completion_tokens == seq.max_tokens:
                 seq.status = SequenceStatus.FINISHED
-                self.cache.release(seq.seq_id)
+                self.release(seq.seq_id)
                 self.running.remove(seq)
                 finished.append(seq)
         return finished

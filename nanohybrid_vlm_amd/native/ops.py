@@ -103,6 +103,7 @@ class NativeBackend:
     library_workspace = 32 << 20  # bytes of scratch memory the library's algorithms may use
     own_kernels_only = False      # True: no library call (matrix products of up to 64 rows take the own kernels)
     planned_context = 0           # > 0 while a HIP graph is recorded: the lengths to plan for (the batch's own are bounds)
+    covered_context = 0           # and the longest context that the recorder will let the graph meet
     measure_linears = False       # True: a product of few rows and a shape not seen before is timed in every way there is (see _choose)
     measure_many_rows = True      # a product of more than library_rows rows is timed in the third step that meets its shape
     measuring_allowed = True      # False: nothing is ever timed; a shape follows the table that was loaded, or the rule
@@ -137,9 +138,13 @@ class NativeBackend:
         return lib
 
     # -- each method launches one kernel; arguments were checked by the caller --
-    def embed(self, ids, table, out):
+    def embed(self, ids, table, out, scale=1.0):
         T, H = out.shape
-        self._call("nhv_embed", _ptr(ids), _ptr(table), _ptr(out), T, H, table.shape[0], dtype_code(table), _stream())
+        self._call("nhv_embed", _ptr(ids), _ptr(table), _ptr(out), T, H, table.shape[0], dtype_code(table),
+                   ctypes.c_float(scale), _stream())
+
+    def soft_cap(self, x, cap):
+        self._call("nhv_soft_cap", _ptr(x), ctypes.c_size_t(x.numel()), ctypes.c_float(cap), _stream())
 
     def rmsnorm(self, x, residual, residual_mode, w, y, eps):
         T, H = x.shape
@@ -156,10 +161,11 @@ class NativeBackend:
                    dtype_code(x), _stream())
 
     def qk_rope_write(self, qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, rot, positions, slot_mapping,
-                      q_out, k_cache, v_cache, Hq, Hkv, D, write_kv):
+                      q_out, k_cache, v_cache, Hq, Hkv, D, write_kv, pair_axes=None):
         wd = dtype_code(q_norm_w) if q_norm_w is not None else dtype_code(qkv)
         self._call("nhv_qk_rope_write", _ptr(qkv), _ptr(bias), _ptr(q_norm_w), _ptr(k_norm_w), ctypes.c_float(eps),
-                   _ptr(cos_sin), rot, 0 if cos_sin is None else cos_sin.shape[0], _ptr(positions), _ptr(slot_mapping),
+                   _ptr(cos_sin), rot, 0 if cos_sin is None else cos_sin.shape[0], _ptr(positions), _ptr(pair_axes),
+                   _ptr(slot_mapping),
                    _ptr(q_out), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], Hq, Hkv, D, int(write_kv),
                    dtype_code(qkv), wd, _stream())
 
@@ -197,12 +203,12 @@ class NativeBackend:
         split_len = 64
         while split_len * 2 <= want and split_len < 1024:
             split_len *= 2
-        # the splits cover the longest context this launch can meet: outside a graph the batch's own; inside one, half
-        # as much again as what was planned for (the recorder replaces a graph before its contexts outgrow that),
-        # not the bound of the block tables (max_model_len), whose splits would nearly all be empty blocks
+        # the splits cover the longest context this launch can meet: outside a graph the batch's own; inside one, what
+        # the recorder says it will let the graph meet (``covered_context``: it replaces a graph before its contexts
+        # outgrow that), not the bound of the block tables (max_model_len), whose splits would nearly all be empty blocks
         covered = batch.max_context_len
-        if self.planned_context:
-            covered = min(covered, self.planned_context + self.planned_context // 2)
+        if self.planned_context and self.covered_context:
+            covered = min(covered, self.covered_context)
         n_splits = -(-covered // split_len)
         part_o = torch.empty((T, Hq, n_splits, D), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, Hq, n_splits, 2), dtype=torch.float32, device=q.device)
@@ -532,14 +538,27 @@ def set_backend(obj) -> None:
 
 
 # ------------------------------------------------------------------ checked entry points
-def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+def embed(ids: torch.Tensor, table: torch.Tensor, scale: float | None = None) -> torch.Tensor:
+    """Rows of ``table``; with ``scale`` each row times it (multiplied in float, rounded once)."""
     _need(table.dim() == 2, "embed: the table must be [vocab, width]")
     _dense(table, "embed: table")
     _dense(ids, "embed: ids", (ids.shape[0],), torch.int32)
     dtype_code(table)
     out = torch.empty((ids.shape[0], table.shape[1]), dtype=table.dtype, device=table.device)
-    backend().embed(ids, table, out)
+    if scale is None:
+        backend().embed(ids, table, out)
+    else:
+        backend().embed(ids, table, out, float(scale))
     return out
+
+
+def soft_cap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place (float32)."""
+    _dense(logits, "soft_cap: logits", dtype=torch.float32)
+    _need(cap > 0, lambda: f"soft_cap: the cap must be positive, got {cap}")
+    if logits.numel():
+        backend().soft_cap(logits, float(cap))
+    return logits
 
 
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, residual: torch.Tensor | None = None,
@@ -594,9 +613,12 @@ def gather_rows(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
 
 
 def qk_rope_write(qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, positions, slot_mapping, k_cache, v_cache,
-                  num_heads: int, num_kv_heads: int, head_dim: int, write_kv: bool = True) -> torch.Tensor:
+                  num_heads: int, num_kv_heads: int, head_dim: int, write_kv: bool = True,
+                  pair_axes: torch.Tensor | None = None) -> torch.Tensor:
     """Splits the packed projection, norms and turns q and k, stores k and v in the
-    paged cache and returns q as [tokens, heads, head_dim]."""
+    paged cache and returns q as [tokens, heads, head_dim].
+    ``positions``: [tokens], or [axes, tokens] with ``pair_axes`` [rotary size / 2] (int32): the axis whose
+    coordinate turns each pair (without ``pair_axes`` every pair turns by the first axis)."""
     T = qkv.shape[0]
     width = (num_heads + 2 * num_kv_heads) * head_dim
     _dense(qkv, "qk_rope_write: qkv", (T, width))
@@ -616,7 +638,16 @@ def qk_rope_write(qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, positions, slot_m
         _dense(cos_sin, "qk_rope_write: rotation table", dtype=torch.float32)
         rot = cos_sin.shape[1]
         _need(rot % 2 == 0 and rot <= head_dim, lambda: f"qk_rope_write: rotary size {rot} with head size {head_dim}")
-    _dense(positions, "qk_rope_write: positions", (T,), torch.int32)
+    if positions.dim() == 1:
+        _dense(positions, "qk_rope_write: positions", (T,), torch.int32)
+    else:
+        _need(positions.dim() == 2 and positions.shape[1] == T and positions.shape[0] >= 1,
+              lambda: f"qk_rope_write: positions {tuple(positions.shape)} for {T} tokens (want [axes, tokens])")
+        _dense(positions, "qk_rope_write: positions", dtype=torch.int32)
+    if pair_axes is not None:
+        _need(cos_sin is not None, "qk_rope_write: axes of pairs without a rotation table")
+        _dense(pair_axes, "qk_rope_write: pair_axes", (rot // 2,), torch.int32)
+        _need(positions.dim() == 2, "qk_rope_write: pair_axes go with positions [axes, tokens]")
     if write_kv:
         _dense(slot_mapping, "qk_rope_write: slot_mapping", (T,), torch.int32)
         _need(k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (num_kv_heads, head_dim),
@@ -626,7 +657,8 @@ def qk_rope_write(qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, positions, slot_m
     q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
     backend().qk_rope_write(qkv, bias, q_norm_w, k_norm_w, float(eps), cos_sin, rot, positions,
                             slot_mapping if write_kv else None, q_out, k_cache if write_kv else None,
-                            v_cache if write_kv else None, num_heads, num_kv_heads, head_dim, write_kv)
+                            v_cache if write_kv else None, num_heads, num_kv_heads, head_dim, write_kv,
+                            **({} if pair_axes is None else {"pair_axes": pair_axes}))
     return q_out
 
 

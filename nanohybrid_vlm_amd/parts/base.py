@@ -7,6 +7,7 @@ architecture's builder turns the configuration into constructor arguments
 """
 from __future__ import annotations
 
+import inspect
 from dataclasses import dataclass, field
 from typing import Callable
 
@@ -116,13 +117,22 @@ class Registry:
     def kinds(self) -> list[str]:
         return sorted(self._makers)
 
-    def build(self, spec: dict, **extra):
-        """``spec`` = {"kind": name, ...constructor arguments}."""
-        spec = dict(spec)
-        kind = spec.pop("kind", None)
+    def maker(self, kind: str):
         if kind not in self._makers:
             raise KeyError(f"unknown {self.what} '{kind}'; registered: {self.kinds()}")
-        return self._makers[kind](**spec, **extra)
+        return self._makers[kind]
+
+    def build(self, spec: dict, offered: dict | None = None, **extra):
+        """``spec`` = {"kind": name, ...constructor arguments}. ``extra``: further arguments that the maker must
+        take. ``offered``: engine options that every part is offered; a maker gets those it names among its
+        parameters (or all of them if it takes ``**kwargs``) and never hears of the others."""
+        spec = dict(spec)
+        maker = self.maker(spec.pop("kind", None))
+        if offered:
+            params = inspect.signature(maker).parameters
+            takes_any = any(p.kind is inspect.Parameter.VAR_KEYWORD for p in params.values())
+            extra = dict({k: v for k, v in offered.items() if (takes_any or k in params) and k not in spec}, **extra)
+        return maker(**spec, **extra)
 
 
 MIXERS = Registry("mixer")

@@ -10,6 +10,10 @@ class PreNormBlock(Part):
     the next norm (nanovllm/models/qwen3.py:152-159): the block takes and returns
     (hidden, residual), and ``residual`` is None before the first block."""
 
+    # the norms this arrangement takes, by the names of its constructor's arguments: the model builds one per slot
+    # from the layer's description (``LayerSpec.norms[slot]``, else ``LayerSpec.norm``)
+    norm_slots = ("mixer_norm", "feed_forward_norm")
+
     def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
         self.mixer = mixer
         self.feed_forward = feed_forward

@@ -24,8 +24,9 @@ class StepContext:
     num_tokens: int
     num_requests: int
     input_ids: torch.Tensor        # [T] int32
-    positions: torch.Tensor        # [T] int32
-    attention: AttentionBatch
+    positions: torch.Tensor        # [axes, T] int32: every token's position as the position encodings see it
+    token_positions: torch.Tensor  # [T] int32: the first axis (all there is for a model of one axis)
+    attention: AttentionBatch      # (its ``positions`` are the tokens' indices in their requests: storage and causality)
     groups: list[GroupTables]
     state_slots: torch.Tensor      # [B] int32: each request's row in the state pools
     logit_rows: torch.Tensor | None  # [n] int32: the tokens whose logits are wanted

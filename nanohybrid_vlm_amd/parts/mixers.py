@@ -61,10 +61,13 @@ class GQAAttention(Part):
     def forward(self, x: torch.Tensor, step, cache: CacheView) -> torch.Tensor:
         tables = step.groups[cache.group]
         qkv = ops.linear(x, self.qkv_weight)
+        # an encoding over several position axes says which axis turns each pair; others turn by the first axis
+        pair_axes = self.position.pair_axes() if hasattr(self.position, "pair_axes") else None
         q = ops.qk_rope_write(
             qkv, self.qkv_bias_t, self.q_norm_weight, self.k_norm_weight,
             self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
-            self.position.rotation_table(), step.positions, tables.slot_mapping, cache.k, cache.v,
-            self.num_heads, self.num_kv_heads, self.head_dim, write_kv=cache.writes)
+            self.position.rotation_table(), step.token_positions if pair_axes is None else step.positions,
+            tables.slot_mapping, cache.k, cache.v, self.num_heads, self.num_kv_heads, self.head_dim,
+            write_kv=cache.writes, pair_axes=pair_axes)
         o = ops.paged_attention(q, cache.k, cache.v, step.attention, tables.block_tables, self.scale, self.window)
         return ops.linear(o.view(o.shape[0], self.num_heads * self.head_dim), self.o_weight)

@@ -18,13 +18,24 @@ from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Cac
 
 @dataclass
 class LayerSpec:
-    """One layer: each entry is {"kind": registered name, ...constructor arguments}."""
+    """One layer: each entry is {"kind": registered name, ...constructor arguments}.
+
+    Which norms a layer has is the block arrangement's affair: a registered block names its norm slots
+    (``norm_slots``, the names of its constructor's arguments) and gets one norm built for each, from
+    ``norms[slot]`` if the layer names that slot, else from ``norm``."""
 
     mixer: dict
     feed_forward: dict
-    norm: dict
+    norm: dict | None = None              # the norm of every slot that ``norms`` does not name
     block: dict = field(default_factory=lambda: {"kind": "prenorm"})
     position: str | None = "default"      # name in ModelSpec.positions that the mixer gets, or None
+    norms: dict = field(default_factory=dict)   # slot name -> {"kind": ..., ...}
+
+    def norm_spec(self, slot: str) -> dict:
+        spec = self.norms.get(slot, self.norm)
+        if spec is None:
+            raise ValueError(f"the layer's block has a norm slot '{slot}' and the layer names no norm for it")
+        return spec
 
 
 @dataclass
@@ -48,6 +59,9 @@ class ModelSpec:
     tie_embeddings: bool
     run_order: list[RunEntry] | None = None   # None: every layer once, in order
     eos_token_id: int | None = None           # the token that ends a request, if the checkpoint names one
+    embed_scale: float | None = None          # the embedding's rows are multiplied by this (in float, then rounded)
+    logit_cap: float | None = None            # logits become cap * tanh(logits / cap)
+    position_axes: int = 1                    # coordinates of a token's position (a step carries [axes, tokens])
 
     def order(self) -> list[RunEntry]:
         if self.run_order is None:
@@ -58,21 +72,31 @@ class ModelSpec:
 class DecoderModel(Part):
     """Embedding, the layers in run order, final norm, and the head on the wanted rows."""
 
-    def __init__(self, spec: ModelSpec):
+    def __init__(self, spec: ModelSpec, options: dict | None = None):
+        """``options``: engine options that are offered to every part's constructor (a part takes those it names,
+        see ``Registry.build``); today ``residual_float32``."""
         self.spec = spec
-        self.positions = {name: POSITION_ENCODINGS.build(p, max_position=spec.max_position)
+        self.options = options = dict(options or {})
+        if spec.position_axes < 1:
+            raise ValueError(f"a model has at least one position axis, got {spec.position_axes}")
+        self.positions = {name: POSITION_ENCODINGS.build(p, offered=options, max_position=spec.max_position)
                           for name, p in spec.positions.items()}
         self.layers = []
         for ls in spec.layers:
             mixer_args = {}
             if ls.position is not None:
                 mixer_args["position"] = self.positions[ls.position]
-            mixer = MIXERS.build(ls.mixer, **mixer_args)
-            ff = FEED_FORWARDS.build(ls.feed_forward)
-            block = BLOCKS.build(ls.block, mixer=mixer, feed_forward=ff,
-                                 mixer_norm=NORMS.build(ls.norm), feed_forward_norm=NORMS.build(ls.norm))
-            self.layers.append(block)
-        self.final_norm = NORMS.build(spec.final_norm)
+            mixer = MIXERS.build(ls.mixer, offered=options, **mixer_args)
+            ff = FEED_FORWARDS.build(ls.feed_forward, offered=options)
+            # the block says which norms it takes; the layer says what each of them is
+            slots = getattr(BLOCKS.maker(ls.block.get("kind")), "norm_slots", ())
+            norms = {slot: NORMS.build(ls.norm_spec(slot), offered=options) for slot in slots}
+            unknown = set(ls.norms) - set(slots)
+            if unknown:
+                raise ValueError(f"the layer names norms {sorted(unknown)}; its block '{ls.block.get('kind')}' has the "
+                                 f"slots {list(slots)}")
+            self.layers.append(BLOCKS.build(ls.block, offered=options, mixer=mixer, feed_forward=ff, **norms))
+        self.final_norm = NORMS.build(spec.final_norm, offered=options)
         self.run_order = spec.order()
         for i, e in enumerate(self.run_order):
             if not 0 <= e.layer < len(self.layers):
@@ -134,7 +158,7 @@ class DecoderModel(Part):
     # -- the forward pass -------------------------------------------------
     def forward(self, step) -> torch.Tensor:
         """Hidden states after the final norm, for the rows whose logits are wanted only: [n, hidden]."""
-        hidden = ops.embed(step.input_ids, self.embed_weight)
+        hidden = ops.embed(step.input_ids, self.embed_weight, self.spec.embed_scale)
         residual = None
         for entry, cache in zip(self.run_order, self.cache_views):
             hidden, residual = self.layers[entry.layer].forward(hidden, residual, step, cache)
@@ -142,10 +166,15 @@ class DecoderModel(Part):
             return None
         # only the wanted rows go through the last norm and the head (nanovllm/layers/embed_head.py:56-61)
         hidden = ops.gather_rows(hidden, step.logit_rows)
+        if residual is None:                  # the last block has made its additions itself
+            return self.final_norm.forward(hidden)
         residual = ops.gather_rows(residual, step.logit_rows)
         hidden, _ = self.final_norm.forward_add(hidden, residual)
         return hidden
 
     def logits(self, hidden: torch.Tensor) -> torch.Tensor:
         """float32 logits [n, vocab] (the reference's sampler casts to float first, nanovllm/layers/sampler.py:12)."""
-        return ops.linear(hidden, self.head_weight, out_dtype=torch.float32)
+        logits = ops.linear(hidden, self.head_weight, out_dtype=torch.float32)
+        if self.spec.logit_cap is not None:
+            ops.soft_cap_(logits, self.spec.logit_cap)
+        return logits

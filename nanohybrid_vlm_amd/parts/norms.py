@@ -12,15 +12,14 @@ class RMSNorm(Part):
     """y = x / sqrt(mean(x^2) + eps) * weight; with a residual the sum is normed
     and carried on (layernorm.py:28-40)."""
 
-    # True: the residual stream is carried in float32 whatever the rows' element type, so the sum goes from layer
-    # to layer unrounded. False: it is carried in the rows' element type, rounded after every addition, as the
-    # reference carries it (layernorm.py:34-40; the norm itself still takes the unrounded float sum). An engine
-    # option, set on every norm of a model by the runner.
-    residual_float32 = True
-
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, residual_float32: bool = True):
+        """``residual_float32`` (an engine option, offered to every part when a model is built): True: the residual
+        stream is carried in float32 whatever the rows' element type, so the sum goes from layer to layer
+        unrounded. False: it is carried in the rows' element type, rounded after every addition, as the
+        reference carries it (layernorm.py:34-40; the norm itself still takes the unrounded float sum)."""
         self.size = size
         self.eps = eps
+        self.residual_float32 = bool(residual_float32)
         self.weight = None
 
     def param_specs(self):

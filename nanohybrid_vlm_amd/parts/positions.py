@@ -1,6 +1,9 @@
 """Position encodings. A position encoding hands the mixer a table of rotation
 angles (cosines and sines per position) or nothing; the mixer's kernel turns
-queries and keys by it before they are used and stored."""
+queries and keys by it before they are used and stored. A token's position may
+have several coordinates (``ModelSpec.position_axes``; a step carries them as
+[axes, tokens]): an encoding over several axes also says, pair by pair, which
+axis' coordinate looks up the pair's angle (``pair_axes``)."""
 from __future__ import annotations
 
 import torch
@@ -8,8 +11,23 @@ import torch
 from .base import POSITION_ENCODINGS, Part
 
 
+class PositionEncoding(Part):
+    """What a mixer asks of its position encoding."""
+
+    def rotation_table(self) -> torch.Tensor | None:
+        """[max_position, rotary_dim] float32 (cosines | sines), or None: nothing is turned."""
+        return None
+
+    def pair_axes(self) -> torch.Tensor | None:
+        """[rotary_dim / 2] int32: the position axis that turns each pair; None: all turn by the first axis."""
+        return None
+
+    def to(self, device):
+        return self
+
+
 @POSITION_ENCODINGS.register("rope")
-class RotaryEmbedding(Part):
+class RotaryEmbedding(PositionEncoding):
     """nanovllm/layers/rotary_embedding.py:83-89: inv_freq_j = base^(-2j/rotary_dim),
     table[p] = [cos(p * inv_freq) | sin(p * inv_freq)] in float32. The rotation
     itself (first half against second half, rotary_embedding.py:6-14) is done by
@@ -37,7 +55,7 @@ class RotaryEmbedding(Part):
 
 
 @POSITION_ENCODINGS.register("none")
-class NoPositions(Part):
+class NoPositions(PositionEncoding):
     """No position signal at all (attention then depends on order only through the mask)."""
 
     def __init__(self, max_position: int, device=None):

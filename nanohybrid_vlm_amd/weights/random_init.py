@@ -86,14 +86,16 @@ def fill_random_on_device(model, seed: int, dtype: torch.dtype, device) -> dict[
     return params
 
 
-def build_random_model(raw_config: dict, seed: int, dtype: str | torch.dtype = "bfloat16", device="cuda:0"):
+def build_random_model(raw_config: dict, seed: int, dtype: str | torch.dtype = "bfloat16", device="cuda:0",
+                       options: dict | None = None):
     """(architecture, typed configuration, model with random weights bound) from config.json contents: what
-    ``ModelRunner`` and ``LLM`` take in place of a model folder. The weights are drawn on the device."""
+    ``ModelRunner`` and ``LLM`` take in place of a model folder. The weights are drawn on the device.
+    ``options``: engine options offered to the parts' constructors (see ``DecoderModel``)."""
     from ..parts.model import DecoderModel
 
     arch = resolve_architecture(raw_config)
     cfg = arch.parse_config(raw_config)
-    model = DecoderModel(arch.build_spec(cfg))
+    model = DecoderModel(arch.build_spec(cfg), options=options)
     if isinstance(dtype, str):
         dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}[dtype]
     fill_random_on_device(model, seed, dtype, device)

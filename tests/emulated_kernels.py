@@ -14,8 +14,12 @@ class EmulatedBackend:
     name = "emulated"
     device_type = "cpu"
 
-    def embed(self, ids, table, out):
-        out.copy_(table[ids.long()])
+    def embed(self, ids, table, out, scale=1.0):
+        rows = table[ids.long()]
+        out.copy_(rows if scale == 1.0 else (rows.float() * scale).to(out.dtype))
+
+    def soft_cap(self, x, cap):
+        x.copy_(cap * torch.tanh(x / cap))
 
     def rmsnorm(self, x, residual, residual_mode, w, y, eps):
         s = x.float()
@@ -35,7 +39,7 @@ class EmulatedBackend:
         out.copy_(x[rows.long()])
 
     def qk_rope_write(self, qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, rot, positions, slot_mapping,
-                      q_out, k_cache, v_cache, Hq, Hkv, D, write_kv):
+                      q_out, k_cache, v_cache, Hq, Hkv, D, write_kv, pair_axes=None):
         T = qkv.shape[0]
         dt = qkv.dtype
         x = qkv.float()
@@ -52,8 +56,15 @@ class EmulatedBackend:
         def turn(t):
             if rot == 0:
                 return t
-            cs = cos_sin[positions.long()]                    # [T, rot]
-            cos, sin = cs[:, None, :rot // 2], cs[:, None, rot // 2:]
+            if positions.dim() == 1:
+                cs = cos_sin[positions.long()]                # [T, rot]
+                cos, sin = cs[:, None, :rot // 2], cs[:, None, rot // 2:]
+            else:
+                # pair j turns by the coordinate of its axis (axis 0 where no axes are named)
+                axes = pair_axes.long() if pair_axes is not None else torch.zeros(rot // 2, dtype=torch.long)
+                at = positions.long()[axes].T                 # [T, rot/2]: the position that turns each pair
+                j = torch.arange(rot // 2)
+                cos, sin = cos_sin[at, j][:, None, :], cos_sin[at, j + rot // 2][:, None, :]
             t1, t2 = t[..., :rot // 2], t[..., rot // 2:rot]
             return torch.cat((t1 * cos - t2 * sin, t2 * cos + t1 * sin, t[..., rot:]), dim=-1)
 

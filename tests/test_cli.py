@@ -92,6 +92,12 @@ def test_bench_program_on_a_tiny_shape():
     assert roofline["bound"] == "hbm" and roofline["peak"] == 8000.0
     assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-3
     assert set(line["points"]) == {"decode_b1", "decode_b64"} and all(v > 0 for v in line["points"].values())
+    # the timed window holds as many steps of GPU work as it counts: with steps issued ahead the mean over the window
+    # and the median of the steps agree (a window that starts after a step issued ahead is done, and ends on a step
+    # that issues none, would be one step short: 20/19 at 20 steps)
+    line, _ = _bench("--shape", "0.6b", "--layers", "8", "--steps", "20", "--warmup", "5", "--batch", "8", "--prompt-tokens",
+                     "512", "--context", "1024", "--no-points", "--no-measured-peaks")
+    assert abs(line["ms_per_step"] - line["step_ms"]["p50"]) / line["step_ms"]["p50"] < 0.05, line
     # a serving workload: every request queued at once, prompts in portions beside decoding requests
     line, _ = _bench("--shape", "tinyB", "--workload", "serving", "--batch", "5", "--prompt-tokens", "150",
                      "--output-tokens", "8", "--block-size", "16", "--no-measured-peaks")

@@ -276,6 +276,9 @@ def test_cache_sized_from_free_memory(model_folders, dtype):
     is right."""
     folder = model_folders["B"]
     cfg, w = plain.read_model_folder(folder)
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()                     # (what earlier tests left in the allocator's reserve goes back: the sizing does the same)
     free_before, total = torch.cuda.mem_get_info()
     share = min(0.9, (total - free_before) / total + 0.04)           # what is in use already and 4 % of the device more
     llm = LLM(folder, dtype=dtype, kvcache_block_size=256, gpu_memory_utilization=share, max_num_batched_tokens=512,
@@ -297,6 +300,21 @@ def test_cache_sized_from_free_memory(model_folders, dtype):
         else:
             _near_best(cfg, w, p, o["token_ids"])
     assert total - torch.cuda.mem_get_info()[0] <= share * total + (256 << 20), "generation stayed within the share (and the allocator's slack)"
+    # what the sizing set aside was measured: after every size of step has been recorded and a step of the whole
+    # token budget (every request wanting logits) has run, the device still holds no more than its share
+    probe = stats["cache_sizing_probe"]
+    assert probe["tokens"] == 512 and probe["activation_bytes"] > 0 and probe["graph_own_bytes"] > 0, probe
+    recorded = llm.warm_up()
+    assert 256 in recorded["graphs_recorded"] and len(recorded["mixed_graphs_recorded"]) >= 9, recorded
+    from nanohybrid_vlm_amd.engine.runner import StepEntry
+    ids = [("full", i) for i in range(min(pages, 300))]
+    budget = [1] * (len(ids) - 1) + [512 - (len(ids) - 1)]
+    llm.runner.step([StepEntry(r, [1] * n, [n - 1]) for r, n in zip(ids, budget)])
+    for r in ids:
+        llm.runner.finish(r)
+    torch.cuda.synchronize()
+    free_now = llm.get_memory_stats()["device_free_bytes"]
+    assert free_now >= (1 - share) * total - (256 << 20), (free_now, (1 - share) * total)
     with pytest.raises(RuntimeError, match="no memory left for the cache"):
         LLM(folder, dtype=dtype, kvcache_block_size=256, gpu_memory_utilization=max(0.001, (total - free_before) / total * 0.5))
 
@@ -405,7 +423,12 @@ def _stress(folder, device, seed, options):
     requests = [(random_tokens(V, rnd_.randint(1, 70), 1000 * seed + i), rnd_.randint(1, 18)) for i in range(36)]
     llm = LLM(folder, dtype="float32", device=device, kvcache_block_size=8, num_kvcache_blocks=rnd_.choice([28, 40, 90]),
               max_num_batched_tokens=rnd_.choice([16, 48, 96]), max_num_seqs=rnd_.choice([4, 9, 36]),
-              max_model_len=96, max_prefill_wait_ms=rnd_.choice([0.0, 1e9]), **options)
+              max_model_len=96, max_prefill_wait_ms=rnd_.choice([0.0, 1e9]),
+              scheduler_policy=rnd_.choice(["decode_first", "prefill_first"]), poison_freed_pages=True, **options)
+    # every slot of the cache that no live request owns holds NaN: all of them now, later every page that a finished
+    # or pushed-out request gives back (the scheduler's releases go through the runner)
+    for kv in llm.runner.kv_tensors:
+        kv.fill_(float("nan"))
     ids, done, waiting = {}, {}, list(enumerate(requests))
     while waiting or not llm.is_finished():
         for _ in range(rnd_.randint(0, 3)):
@@ -435,3 +458,31 @@ def test_engine_under_random_arrivals_on_gpu(model_folders, seed):
     llm, stats = _stress(model_folders["B"], "cuda:0", seed, dict(max_graph_tokens=64))
     assert not stats["graphs_refused"] and not stats["mixed_graphs_refused"]
     assert stats["graphs_recorded"] and stats["mixed_graphs_recorded"], stats
+
+
+def test_end_token_from_the_tokenizer_and_text_prompts(emulated_kernels, tmp_path):
+    """A model folder whose config.json names no end token ends requests where its tokenizer does
+    (nanovllm/engine/llm_engine.py:207-223); with a tokenizer.json a prompt may be text and the answer comes as text too."""
+    import json
+    from conftest import TINY_C
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    from nanohybrid_vlm_amd.weights.random_init import write_random_model
+    folder = write_random_model(str(tmp_path / "m"), TINY_C, seed=2)
+    assert "eos_token_id" not in TINY_C
+    vocab = {f"w{i}": i for i in range(TINY_C["vocab_size"] - 1)}
+    vocab["<end>"] = TINY_C["vocab_size"] - 1
+    tok = Tokenizer(models.WordLevel(vocab, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.save(str(tmp_path / "m" / "tokenizer.json"))
+    options = dict(dtype="float32", device="cpu", kvcache_block_size=8, num_kvcache_blocks=16, max_model_len=64)
+    assert LLM(folder, **options).config.eos == -1                   # a tokenizer alone does not say which token ends
+    (tmp_path / "m" / "tokenizer_config.json").write_text(json.dumps({"eos_token": {"content": "<end>"}}))
+    llm = LLM(folder, **options)
+    assert llm.config.eos == TINY_C["vocab_size"] - 1
+    out = llm.generate(["w5 w17 w3"], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True), use_tqdm=False)[0]
+    cfg, w = plain.read_model_folder(folder)
+    assert out["token_ids"] == plain.greedy_generate(cfg, w, [5, 17, 3], 4)
+    assert out["text"] == tok.decode(out["token_ids"])
+    (tmp_path / "m" / "tokenizer_config.json").write_text(json.dumps({"eos_token": "w9"}))
+    assert LLM(folder, eos=4, **options).config.eos == 4              # an end token that the caller names stands
+    assert LLM(folder, **options).config.eos == 9

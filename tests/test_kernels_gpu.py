@@ -241,6 +241,52 @@ def test_qk_rope_write(ops, dtype, Hq, Hkv, D, rot, norm, bias):
     assert not kf[untouched].any() and not vf[untouched].any()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,rot,axes", [(4, 2, 16, 16, 2), (3, 1, 48, 24, 3), (8, 2, 128, 128, 2), (2, 2, 32, 8, 1)])
+def test_qk_rope_write_over_several_position_axes(ops, dtype, Hq, Hkv, D, rot, axes):
+    """positions [axes, T]: pair j of a head turns by the angle that the table holds at the coordinate of axis
+    pair_axes[j] (without pair_axes: of the first axis)."""
+    from nanohybrid_vlm_amd.parts.positions import RotaryEmbedding
+    T, base = 19, 10000.0
+    width = (Hq + 2 * Hkv) * D
+    qkv = rnd(T, width, dtype=dtype, seed=19, scale=2.0)
+    table = RotaryEmbedding(rot, 200, base).table.cuda()
+    positions = torch.randint(0, 200, (axes, T), dtype=torch.int32, device="cuda")
+    pair_axes = (torch.arange(rot // 2) * 5 % axes).to(torch.int32).cuda() if axes > 1 else None
+    slots = torch.arange(T, dtype=torch.int32, device="cuda")
+    k_cache = torch.zeros(4, 8, Hkv, D, dtype=dtype, device="cuda")
+    v_cache = torch.zeros_like(k_cache)
+    q = ops.qk_rope_write(qkv, None, None, None, 0.0, table, positions, slots, k_cache, v_cache, Hq, Hkv, D, pair_axes=pair_axes)
+    # the angle of pair j at position p is p * base^(-2j/rot): here p differs from pair to pair
+    j = torch.arange(rot // 2)
+    at = positions.cpu().long()[pair_axes.cpu().long() if pair_axes is not None else torch.zeros(rot // 2, dtype=torch.long)].T   # [T, rot/2]
+    ang = at.double() * (base ** (-2.0 * j.double() / rot))
+    cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+
+    def turned(x):
+        x = x.double().cpu()
+        x1, x2 = x[..., :rot // 2], x[..., rot // 2:rot]
+        return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., rot:]), -1)
+
+    x = qkv.float()
+    t = dict(rtol=1.6e-2, atol=1.6e-2) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(q.double().cpu(), turned(x[:, :Hq * D].reshape(T, Hq, D)), **t)
+    torch.testing.assert_close(k_cache.view(-1, Hkv, D)[:T].double().cpu(), turned(x[:, Hq * D:(Hq + Hkv) * D].reshape(T, Hkv, D)), **t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_scale_and_soft_cap(ops, dtype):
+    table = rnd(301, 200, dtype=dtype, seed=21)
+    ids = torch.randint(0, 301, (13,), dtype=torch.int32, device="cuda")
+    assert torch.equal(ops.embed(ids, table, 1.0), table[ids.long()])
+    assert torch.equal(ops.embed(ids, table, 1.75), (table[ids.long()].float() * 1.75).to(dtype))
+    logits = rnd(7, 1001, seed=22, scale=6.0)
+    want = 4.0 * torch.tanh(logits / 4.0)
+    assert ops.soft_cap_(logits, 4.0) is logits
+    torch.testing.assert_close(logits, want, rtol=1e-5, atol=1e-5)
+    assert float(logits.abs().max()) <= 4.0
+
+
 def _paged_setup(dtype, lens, q_lens, Hq, Hkv, D, page, seed=0, scale=1.0):
     """Requests with ``lens`` keys each whose last ``q_lens`` tokens are this step's queries; pages handed out
     in a shuffled order. Returns the pieces for ops.paged_attention and the dense keys and values."""

@@ -58,6 +58,25 @@ def _toy_check(device, dtype, tol, tmp_path, device_state=False, graphs=False):
         if runner.use_graphs and mode in ("tail", "mixed"):
             stats = runner.get_memory_stats()
             assert stats["graphs_recorded"] and not stats["graphs_refused"], stats
+    # positions of the requests' own on the second axis (the first stays the index): every way of cutting again
+    second_axis = {rid: [(5 * i + 3) % 11 + i // 3 for i in range(len(toks))] for rid, toks in requests.items()}
+    want = {rid: toy_plain_logits(w, toks, positions=[list(range(len(toks))), second_axis[rid]])
+            for rid, toks in requests.items()}
+    for mode, steps in [("portions", rc.portions(requests)), ("tail", rc.tail_decoded(requests, tail=12)),
+                        ("mixed", rc.mixed(requests, max_live=3))]:
+        fed = {rid: 0 for rid in requests}
+        for st in steps:
+            for e in st["entries"]:
+                a, b = fed[e["id"]], fed[e["id"]] + len(e["tokens"])
+                e["positions"] = [list(range(a, b)), second_axis[e["id"]][a:b]]
+                fed[e["id"]] = b
+        pages = rc.peak_tokens(steps, 4) // 4
+        runner = ModelRunner(folder, dtype=dtype, device=device, page_size=4, num_pages=pages, num_state_slots=3,
+                             use_graphs=graphs, max_model_len=64)
+        got = rc.run_in_process(runner, steps)
+        for rid in requests:
+            d = max_abs_diff(got[rid], want[rid])
+            assert d <= tol, f"toy with positions of its own, {mode}: request {rid}: {d:.3e}"
     # the windowed group gives pages back while a request is still alive
     runner = ModelRunner(folder, dtype=dtype, device=device, page_size=4, num_pages=16, num_state_slots=3)
     runner.step([StepEntry("x", requests["r1"][:30], [29])])

@@ -118,3 +118,66 @@ def test_graph_buckets_are_powers_of_two_and_the_sizes_half_way_up_to_the_limit(
         runner = ModelRunner(model_folders["A"], dtype="float32", device="cpu", page_size=4, num_pages=8, num_state_slots=2,
                              max_graph_batch=limit)
         assert runner.graph_buckets == want
+
+
+def test_a_recorded_short_step_is_strictly_smaller_than_its_bucket(model_folders, emulated_kernels, tmp_path):
+    """A short step of prompt portions is padded to a bucket of tokens by one more request that owns the filling
+    tokens. The bucket is strictly larger than the step, so that request has at least one token, and every request
+    of the padded batch, also the ones without tokens, has its first row inside the batch: a part that works from the
+    step's device tensors may index rows by ``cu_seqlens_q[:-1]`` (the toy's state mixer does)."""
+    import torch
+    import toy_architecture as toy
+    from nanohybrid_vlm_amd.weights.random_init import write_random_model
+    runner = ModelRunner(model_folders["A"], dtype="float32", device="cpu", page_size=4, num_pages=40, num_state_slots=4)
+    runner.use_graphs, runner.max_graph_tokens, runner.mixed_token_buckets = True, 24, [16, 24]
+    met = []
+    runner._mixed_graph_step = lambda entries, key, keep=True: met.append(key)
+    runner.step([StepEntry("a", list(range(15)), [14])])
+    runner.step([StepEntry("b", list(range(16)), [15])])                      # fills the bucket of 16: goes to 24
+    assert met == [(16, 1), (24, 1)]
+    assert runner.step([StepEntry("c", list(range(24)), [23])]).shape == (1, runner.vocab_size)   # no bucket above: eager
+    # the layout of such a step, and the toy's state mixer on it
+    toy.register()
+    try:
+        folder = write_random_model(str(tmp_path / "toy"), {"architectures": ["ToyForCausalLM"], "model_type": "toy",
+                                                            "device_state": True}, seed=4)
+        runner = ModelRunner(folder, dtype="float32", device="cpu", page_size=4, num_pages=40, num_state_slots=4)
+        entries = [StepEntry("a", list(range(9)), [8]), StepEntry("b", list(range(6)), [])]
+        arrays, meta = runner._layout(entries, pad_to=4, table_width=16, pad_tokens_to=16)
+        cu = arrays[3]
+        assert meta["T"] == 16 and meta["B"] == 5 and list(cu) == [0, 9, 15, 15, 15, 16]
+        assert (cu[:-1] < meta["T"]).all()
+        dev = [torch.from_numpy(a) for a in arrays]
+        ctx = runner._context(dev, meta, None, 0, max_context_len=64)
+        assert ctx.positions.shape == (toy.AXES, 16) and ctx.token_positions.shape == (16,)
+        runner.model.forward(ctx)                                              # (no row index runs out of the batch)
+    finally:
+        toy.unregister()
+
+
+def test_positions_of_several_axes(model_folders, emulated_kernels, tmp_path):
+    """A model of one position axis carries no array of positions unless an entry brings its own; a model of two
+    axes always carries [2, T]: the tokens' indices on both axes, or what the entry says."""
+    import toy_architecture as toy
+    from nanohybrid_vlm_amd.weights.random_init import write_random_model
+    runner = ModelRunner(model_folders["A"], dtype="float32", device="cpu", page_size=4, num_pages=40, num_state_slots=4)
+    arrays, _ = runner._layout([StepEntry("a", [1, 2, 3], [])])
+    assert len(arrays) == 8
+    runner.cache.commit("a", 3)
+    arrays, _ = runner._layout([StepEntry("a", [4, 5], [], positions=[[9, 11]]), StepEntry("b", [6], [])])
+    assert len(arrays) == 9 and arrays[8].tolist() == [[9, 11, 0]] and arrays[1].tolist() == [3, 4, 0]
+    with pytest.raises(ValueError, match=r"positions must be \[1\]\[2\]"):
+        runner._layout([StepEntry("c", [4, 5], [], positions=[[1, 2], [3, 4]])])
+    with pytest.raises(ValueError, match="outside the model's"):
+        runner._layout([StepEntry("c", [4, 5], [], positions=[[1, runner.max_position]])])
+    toy.register()
+    try:
+        folder = write_random_model(str(tmp_path / "toy"), {"architectures": ["ToyForCausalLM"], "model_type": "toy"}, seed=4)
+        runner = ModelRunner(folder, dtype="float32", device="cpu", page_size=4, num_pages=40, num_state_slots=4)
+        arrays, _ = runner._layout([StepEntry("a", [1, 2, 3], [])])
+        assert arrays[-1].tolist() == [[0, 1, 2], [0, 1, 2]]
+        runner.cache.commit("a", 3)
+        arrays, _ = runner._layout([StepEntry("a", [4], [0], positions=[[3], [7]]), StepEntry("b", [5], [0])], pad_to=4, table_width=8)
+        assert arrays[-1].tolist() == [[3, 0, 0, 0], [7, 0, 0, 0]]
+    finally:
+        toy.unregister()

@@ -91,3 +91,41 @@ def test_no_alloc_entry_point_refuses_what_does_not_fit():
     assert rc == 0, lib.nhv_last_error().decode()
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all() and out.any()
+
+
+def test_no_alloc_entry_point_recorded_into_a_graph():
+    """After the address of the array is known on the device (``nhv_decode_attention_no_alloc_init``, outside any
+    capture) a call only launches kernels: it is recorded into a HIP graph and replayed, with other work between
+    the replays and with other inputs in the same buffers, and gives the existing entry point's result each time."""
+    Hq, Hkv, D, page, split_len = 8, 2, 128, 64, 128
+    lib = _library(D)
+    assert lib.nhv_decode_attention_no_alloc_init() == 0, lib.nhv_last_error().decode()
+    lens = [900, 130, 64, 513]
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, [1] * len(lens), Hq, Hkv, D, page, seed=11, scale=1.5)
+    T, n_splits = len(lens), -(-max(lens) // split_len)
+    scale = ctypes.c_float(D ** -0.5)
+    got = torch.zeros_like(q)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        rc = lib.nhv_decode_attention_bf16_no_alloc(_p(q), _p(kc), _p(vc), _p(got), _p(batch.token_req), _p(batch.positions),
+                                                    _p(bt), bt.shape[1], T, Hq, Hkv, page, scale, 0, split_len, n_splits,
+                                                    ctypes.c_void_p(side.cuda_stream))
+    assert rc == 0, lib.nhv_last_error().decode()
+    part_o = torch.empty((T, Hq, n_splits, D), dtype=torch.float32, device="cuda")
+    part_ml = torch.empty((T, Hq, n_splits, 2), dtype=torch.float32, device="cuda")
+    for replay in range(3):
+        if replay:
+            q.copy_(torch.randn_like(q.float()).to(q.dtype))          # other queries in the same buffer
+        want = torch.empty_like(q)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.nhv_decode_attention_bf16(_p(q), _p(kc), _p(vc), _p(want), _p(part_o), _p(part_ml), _p(batch.token_req),
+                                           _p(batch.positions), _p(bt), bt.shape[1], T, Hq, Hkv, page, scale, 0, split_len,
+                                           n_splits, stream)
+        assert rc == 0, lib.nhv_last_error().decode()
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {replay}"

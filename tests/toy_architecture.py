@@ -3,8 +3,11 @@ keeps state of its own per request (in two versions: one that loops over the ste
 requests on the host, and one that works from the step's device tensors alone and can
 therefore be recorded into a graph), a feed-forward that routes every token to one of
 several experts, a position encoding of its own (other angles, on a part of the head
-only), a layer with a window, a layer that runs twice and an entry that reads another
-entry's cache; and its plain whole-sequence computation.
+only, over two position axes: even pairs turn by the first coordinate of a token's
+position, odd pairs by the second), a block arrangement of its own with a third norm
+after the mixer (of another eps than the layer's other norms), an embedding scale and a
+cap on the logits, a layer with a window, a layer that runs twice and an entry that
+reads another entry's cache; and its plain whole-sequence computation.
 
 Importing this module registers the parts and the architecture (so the command line can
 take it as ``--plugin toy_architecture``); ``unregister()`` takes them out again.
@@ -18,11 +21,12 @@ import torch
 import plain_qwen3 as plain
 from nanohybrid_vlm_amd.config.registry import (Architecture, WeightSource, register_architecture,
                                                 unregister_architecture)
-from nanohybrid_vlm_amd.parts import FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, ParamSpec, Part, StateNeed
+from nanohybrid_vlm_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, ParamSpec, Part, StateNeed
 from nanohybrid_vlm_amd.parts.model import DecoderModel, LayerSpec, ModelSpec, RunEntry
 
 H, HEADS, KV, D, INTER, VOCAB, WINDOW, DECAY = 48, 3, 1, 16, 64, 97, 5, 0.75
 EXPERTS, EXPERT_INTER, TOY_ROT, TOY_STEP = 3, 40, 8, 0.05
+AXES, EMBED_SCALE, LOGIT_CAP, POST_EPS = 2, 1.75, 4.0, 1e-2
 
 
 class DecayingSum(Part):
@@ -70,7 +74,7 @@ class DecayingSumOnDevice(DecayingSum):
         pool = cache.state["sum"]
         batch = step.attention
         req = batch.token_req.long()
-        pos = step.positions.to(torch.float64)
+        pos = batch.positions.to(torch.float64)                         # the tokens' indices in their requests
         first_row = batch.cu_seqlens_q[:-1].long()                      # [B] row of every request's first token
         last_row = batch.cu_seqlens_q[1:].long() - 1
         slots = step.state_slots.long()
@@ -131,19 +135,50 @@ class RoutedFeedForward(Part):
 
 
 class LinearAngles(Part):
-    """Toy position encoding: the angle of pair j at position p is p * (j + 1) * step, and only the first
-    ``rotary_dim`` entries of a head are turned."""
+    """Toy position encoding: the angle of pair j at position p is p * (j + 1) * step, only the first
+    ``rotary_dim`` entries of a head are turned, and p is the coordinate of axis j % axes of the token's position."""
 
-    def __init__(self, rotary_dim: int, step: float, max_position: int, device=None):
+    def __init__(self, rotary_dim: int, step: float, max_position: int, axes: int = 1, device=None):
         ang = torch.arange(max_position, dtype=torch.float32)[:, None] * (torch.arange(rotary_dim // 2) + 1.0) * step
         self.table = torch.cat((ang.cos(), ang.sin()), dim=-1).contiguous()
+        self.axes = (torch.arange(rotary_dim // 2) % axes).to(torch.int32) if axes > 1 else None
 
     def rotation_table(self):
         return self.table
 
+    def pair_axes(self):
+        return self.axes
+
     def to(self, device):
         self.table = self.table.to(device)
+        if self.axes is not None:
+            self.axes = self.axes.to(device)
         return self
+
+
+class SandwichBlock(Part):
+    """Toy block arrangement with three norms: r += post_mixer_norm(mixer(mixer_norm(r))); r += feed_forward(
+    feed_forward_norm(r)). It keeps the engine's convention of (hidden, residual) with the second addition left to
+    the next norm."""
+
+    norm_slots = ("mixer_norm", "post_mixer_norm", "feed_forward_norm")
+
+    def __init__(self, mixer, feed_forward, mixer_norm, post_mixer_norm, feed_forward_norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.post_mixer_norm, self.feed_forward_norm = mixer_norm, post_mixer_norm, feed_forward_norm
+
+    def children(self):
+        return {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "post_mixer_norm": self.post_mixer_norm,
+                "feed_forward_norm": self.feed_forward_norm, "feed_forward": self.feed_forward}
+
+    def forward(self, hidden, residual, step, cache):
+        if residual is None:
+            x, residual = self.mixer_norm.forward_start(hidden)
+        else:
+            x, residual = self.mixer_norm.forward_add(hidden, residual)
+        x = self.post_mixer_norm.forward(self.mixer.forward(x, step, cache))
+        x, residual = self.feed_forward_norm.forward_add(x, residual)
+        return self.feed_forward.forward(x, step), residual
 
 
 def toy_spec(cfg: dict) -> ModelSpec:
@@ -157,7 +192,8 @@ def toy_spec(cfg: dict) -> ModelSpec:
     routed = {"kind": "toy_routed", "hidden_size": H, "intermediate_size": EXPERT_INTER, "num_experts": EXPERTS,
               "on_device": bool(cfg.get("device_state"))}
     layers = [
-        LayerSpec(mixer=attention(None), feed_forward=ff, norm=norm),
+        LayerSpec(mixer=attention(None), feed_forward=ff, norm=norm, block={"kind": "toy_sandwich"},
+                  norms={"post_mixer_norm": {"kind": "rmsnorm", "size": H, "eps": POST_EPS}}),
         LayerSpec(mixer={"kind": state_mixer, "hidden_size": H, "decay": DECAY}, feed_forward=routed, norm=norm),
         LayerSpec(mixer=attention(None if cfg.get("no_window") else WINDOW), feed_forward=ff, norm=norm, position="linear"),
     ]
@@ -165,8 +201,9 @@ def toy_spec(cfg: dict) -> ModelSpec:
     order = [RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(2, cache=2)]
     return ModelSpec(vocab_size=VOCAB, hidden_size=H, layers=layers, final_norm=norm,
                      positions={"default": {"kind": "rope", "rotary_dim": D, "base": 1000.0},
-                                "linear": {"kind": "toy_linear_angles", "rotary_dim": TOY_ROT, "step": TOY_STEP}},
-                     max_position=256, tie_embeddings=True, run_order=order, eos_token_id=cfg.get("eos_token_id"))
+                                "linear": {"kind": "toy_linear_angles", "rotary_dim": TOY_ROT, "step": TOY_STEP, "axes": AXES}},
+                     max_position=256, tie_embeddings=True, run_order=order, eos_token_id=cfg.get("eos_token_id"),
+                     embed_scale=EMBED_SCALE, logit_cap=LOGIT_CAP, position_axes=AXES)
 
 
 def toy_names(cfg):
@@ -174,23 +211,28 @@ def toy_names(cfg):
 
 
 def toy_turn(x, pos):
-    """The toy position encoding on [T, heads, D]: pairs (j, j + TOY_ROT / 2) of the first TOY_ROT entries."""
-    ang = pos.float()[:, None] * (torch.arange(TOY_ROT // 2) + 1.0) * TOY_STEP
+    """The toy position encoding on [T, heads, D]: pairs (j, j + TOY_ROT / 2) of the first TOY_ROT entries; pair j
+    turns by the coordinate of axis j % AXES (``pos``: [AXES, T])."""
+    j = torch.arange(TOY_ROT // 2)
+    ang = pos.float()[j % AXES].T * (j + 1.0) * TOY_STEP
     cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
     x1, x2 = x[..., :TOY_ROT // 2], x[..., TOY_ROT // 2:TOY_ROT]
     return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., TOY_ROT:]), dim=-1)
 
 
-def toy_plain_logits(w, toks, no_window=False):
-    """Whole sequence, no cache, from the plain functions."""
+def toy_plain_logits(w, toks, no_window=False, positions=None):
+    """Whole sequence, no cache, from the plain functions. ``positions``: [AXES, T] coordinates for the encoding
+    over several axes (default: the tokens' indices on every axis)."""
     window_of_layer_2 = None if no_window else WINDOW
     T = len(toks)
     pos = torch.arange(T)
-    r = w["embed.weight"][toks]
+    axes_pos = torch.stack([pos] * AXES) if positions is None else torch.as_tensor(positions)
+    r = w["embed.weight"][toks] * EMBED_SCALE
     kept = {}
 
     def attention(x, p, window, entry, lender=None):
-        turn = toy_turn if p.startswith("layers.2.") else (lambda t, at: plain.apply_rope(t, at, 1000.0))   # layer 2 has the toy angles
+        # layer 2 has the toy angles over both axes; the other layers' rotation takes the first axis, the index
+        turn = (lambda t, at: toy_turn(t, axes_pos)) if p.startswith("layers.2.") else (lambda t, at: plain.apply_rope(t, at, 1000.0))
         qkv = x @ w[p + "mixer.qkv.weight"].T
         q = plain.rms_norm(qkv[:, :HEADS * D].view(T, HEADS, D), w[p + "mixer.q_norm.weight"], 1e-5)
         if lender is None:
@@ -223,19 +265,23 @@ def toy_plain_logits(w, toks, no_window=False):
         x = plain.rms_norm(r, w[p + "mixer_norm.weight"], 1e-5)
         if layer == 1:
             r = r + decaying_sum(x, p)
+        elif layer == 0:                     # the sandwich block: a norm of its own after the mixer
+            r = r + plain.rms_norm(attention(x, p, None, entry, lender), w[p + "post_mixer_norm.weight"], POST_EPS)
         else:
-            r = r + attention(x, p, window_of_layer_2 if layer == 2 else None, entry, lender)
+            r = r + attention(x, p, window_of_layer_2, entry, lender)
         x = plain.rms_norm(r, w[p + "feed_forward_norm.weight"], 1e-5)
         if layer == 1:
             r = r + routed(x, p)
             continue
         gu = w[p + "feed_forward.gate_up.weight"]
         r = r + plain.swiglu(x, gu[:INTER], gu[INTER:], w[p + "feed_forward.down.weight"])
-    return plain.rms_norm(r, w["final_norm.weight"], 1e-5) @ w["embed.weight"].T
+    logits = plain.rms_norm(r, w["final_norm.weight"], 1e-5) @ w["embed.weight"].T
+    return LOGIT_CAP * torch.tanh(logits / LOGIT_CAP)
 
 
 _PARTS = [(MIXERS, "toy_decaying_sum", DecayingSum), (MIXERS, "toy_decaying_sum_on_device", DecayingSumOnDevice),
-          (FEED_FORWARDS, "toy_routed", RoutedFeedForward), (POSITION_ENCODINGS, "toy_linear_angles", LinearAngles)]
+          (FEED_FORWARDS, "toy_routed", RoutedFeedForward), (POSITION_ENCODINGS, "toy_linear_angles", LinearAngles),
+          (BLOCKS, "toy_sandwich", SandwichBlock)]
 
 
 def register_parts() -> None:
