@@ -46,6 +46,7 @@ def parse_args():
     ap.add_argument("--prompt-tokens", type=int, default=None, help="8b: 2048; 32b: 8192; 14b: the longest prompt, 4096")
     ap.add_argument("--output-tokens", type=int, default=None, help="14b: 128; 32b: 256")
     ap.add_argument("--context", type=int, default=None, help="max_model_len (8b: 4096)")
+    ap.add_argument("--token-budget", type=int, default=2048, help="tokens in one step (max_num_batched_tokens): a prompt longer than this is fed in portions")
     ap.add_argument("--block-size", type=int, default=256)
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 runs")
@@ -54,6 +55,8 @@ def parse_args():
     ap.add_argument("--max-graph-batch", type=int, default=None, help="largest decode batch that replays a graph")
     ap.add_argument("--residual-dtype", default="float32", choices=("float32", "model"),
                     help="the residual stream between layers: float32, or rounded to the element type as the reference does")
+    ap.add_argument("--no-fuse-norms", action="store_true",
+                    help="products of few rows leave the residual addition and the norm to kernels of their own")
     ap.add_argument("--gemm-choices", default=None, help="JSON file of matrix-product choices to follow (and to write if absent)")
     return ap.parse_args()
 
@@ -75,6 +78,7 @@ def build_llm(args, max_seqs, **options):
         raw["num_hidden_layers"] = args.layers
     llm = LLM(raw, random_weights=0, dtype=args.dtype, kvcache_block_size=args.block_size, max_num_seqs=max_seqs,
               enforce_eager=args.eager, gemm_choices=args.gemm_choices, residual_dtype=args.residual_dtype,
+              fuse_norms=not args.no_fuse_norms,
               **({"max_graph_batch": args.max_graph_batch} if args.max_graph_batch else {}), **options)
     return llm, llm.runner.cfg, full_layers
 
@@ -187,7 +191,7 @@ def bench_decode_points(args):
     max_seqs = max(batch, 1 if args.no_points else 64)
     pages_per_seq = -(-context // args.block_size)
     llm, cfg, full_layers = build_llm(args, max_seqs, num_kvcache_blocks=max_seqs * pages_per_seq + 1,
-                                      max_num_batched_tokens=max(2048, max_seqs), max_model_len=context,
+                                      max_num_batched_tokens=max(args.token_budget, max_seqs), max_model_len=context,
                                       scheduler_policy="prefill_first")   # while prompts are fed nothing decodes, so all requests decode in step
     weight_bytes, kv_per_token, matrix_flops = model_bytes_and_flops(cfg, itemsize)
     peaks = measured_peaks(args)
@@ -253,7 +257,7 @@ def bench_workload(args):
         context = args.context or (longest + n_out)
         pages = sum(-(-(n + n_out) // args.block_size) for n in lengths) + 1
         cache = {"num_kvcache_blocks": pages}
-        workload = f"{batch} requests, prompts uniform in [128, {longest}], {n_out} new tokens each, portions of 2048"
+        workload = f"{batch} requests, prompts uniform in [128, {longest}], {n_out} new tokens each, portions of {args.token_budget}"
     else:
         batch, n_out = args.batch or 16, args.output_tokens or 256
         longest = args.prompt_tokens or 8192
@@ -261,7 +265,7 @@ def bench_workload(args):
         context = args.context or (longest + n_out)
         cache = {"num_kvcache_blocks": -1}            # the cache takes what is left of the device's memory
         workload = f"{batch} requests of {longest} prompt tokens, {n_out} new tokens each, cache sized from free memory"
-    llm, cfg, full_layers = build_llm(args, batch, max_num_batched_tokens=2048, max_model_len=context, **cache)
+    llm, cfg, full_layers = build_llm(args, batch, max_num_batched_tokens=args.token_budget, max_model_len=context, **cache)
     weight_bytes, kv_per_token, matrix_flops = model_bytes_and_flops(cfg, itemsize)
     peaks = measured_peaks(args)
     sp = SamplingParams(temperature=0.0, max_tokens=n_out, ignore_eos=True)
@@ -298,7 +302,7 @@ def bench_workload(args):
         "ms_per_step": round(wall / len(steps) * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dname, "data": "synthetic: random token ids, random weights N(0, 0.02^2), norms 1 + N(0, 0.1^2)",
         "config": config_of(args, cfg, full_layers, global_batch=batch, prompt_len=longest, seq_len=context,
-                            token_budget=2048, cache_pages=stats["groups"][0]["pages"]),
+                            token_budget=args.token_budget, cache_pages=stats["groups"][0]["pages"]),
         "prefill": {"value": round(prompt_tokens / prompt_s, 1) if prompt_s else None, "tokens": sum(lengths),
                     "ms": round(prompt_s * 1e3, 3), "frac": round(matrix_flops * prompt_tokens / prompt_s / PEAK_FLOPS[dname], 4) if prompt_s else None},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

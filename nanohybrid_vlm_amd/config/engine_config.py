@@ -36,6 +36,7 @@ class EngineConfig:
     # once per shape and process; which way wins can differ from start to start, and with it the last bits of the logits.
     measure_gemms: bool = True                  # False: nothing is timed; shapes follow gemm_choices, else the fixed rule
     gemm_choices: str | None = None             # a JSON file of choices: read if it exists (and then nothing is timed), see LLM.save_gemm_choices
+    fuse_norms: bool = True                     # bfloat16 products of up to 16 rows make the residual addition after them and the norm before them in their own kernels
     dtype: str = "bfloat16"                     # "bfloat16" or "float32" (true 32-bit everywhere)
     # the residual stream between layers in a bfloat16 run: "float32" keeps the unrounded sum; "model" rounds it to
     # bfloat16 after every addition, as the reference does (and reads and writes a third fewer bytes in every norm)

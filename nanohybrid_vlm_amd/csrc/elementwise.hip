@@ -482,3 +482,25 @@ extern "C" int nhv_qk_rope_write(const void* qkv, const void* bias, const void* 
   NHV_LAUNCH_CHECK("qk_rope_write");
   return 0;
 }
+
+// ---------------------------------------------------------------- rows' scales applied on their own
+// y[m][k] = round(x[m][k] * r[m]), r[m] = 1 / sqrt(sum over tiles of ss[m][.] / H + eps): what a few-rows product
+// does in its own kernel for a sum whose norm is due (nhv_gemm_fusion.h), for a reader that is no such product.
+__global__ void scale_rows_kernel(const bf16_t* __restrict__ x, const float* __restrict__ ss, int tiles, float eps,
+                                  bf16_t* __restrict__ y, int H) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  float sum = 0.f;
+  for (int t = threadIdx.x; t < tiles; t += blockDim.x) sum += ss[(size_t)m * tiles + t];
+  const float total = block_sum(sum, scratch);
+  const float r = 1.0f / sqrtf(total / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) y[(size_t)m * H + i] = (bf16_t)((float)x[(size_t)m * H + i] * r);
+}
+
+extern "C" int nhv_scale_rows(const void* x, const void* ss, int tiles, float eps, void* y, int M, int H, void* stream) {
+  NHV_REQUIRE(M > 0 && H > 0 && tiles > 0, "scale_rows: bad sizes M=%d H=%d tiles=%d", M, H, tiles);
+  hipLaunchKernelGGL(scale_rows_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (const float*)ss, tiles,
+                     eps, (bf16_t*)y, H);
+  NHV_LAUNCH_CHECK("scale_rows");
+  return 0;
+}

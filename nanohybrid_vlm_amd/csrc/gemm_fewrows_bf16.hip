@@ -24,8 +24,11 @@
 // K over several blocks, with the last one to arrive adding the parts in order, was measured and never
 // won: the fences cost more than the balance gains.)
 #include "nhv_common.h"
+#include "nhv_gemm_fusion.h"
 
 namespace fewrows {
+
+typedef NhvGemmFusion Fusion;
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -38,19 +41,118 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// The scales of the rows of an x whose norm is still due (nhv_gemm_fusion.h), in two steps, so that the wait for
+// the shares falls where other loads are under way. ask_row_scales: wave w asks for the shares of rows w, w + WAVES,
+// ... (M <= 16: SCALE_ROWS<WAVES> rows at most), SCALE_SHARES of them per lane and row. set_row_scales: adds them up
+// in a fixed order and leaves the scales in r_s[0..M); the caller's next barrier makes them visible.
+constexpr int SCALE_SHARES = 4;              // up to 256 tiles (rows of 4,096) in one go; what is beyond is read when the sums are made
+template <int WAVES>
+constexpr int SCALE_ROWS = (16 + WAVES - 1) / WAVES;
+template <int WAVES>
+__device__ __forceinline__ void ask_row_scales(const Fusion& f, float (&share)[SCALE_ROWS<WAVES>][SCALE_SHARES], int M, int wave, int lane) {
+  if (f.ss_in == nullptr) return;
+#pragma unroll
+  for (int i = 0; i < SCALE_ROWS<WAVES>; ++i) {
+    const int m = wave + i * WAVES;
+#pragma unroll
+    for (int j = 0; j < SCALE_SHARES; ++j) {
+      const int t = lane + j * 64;
+      share[i][j] = (m < M && t < f.tiles_in) ? f.ss_in[(size_t)m * f.tiles_in + t] : 0.f;
+    }
+  }
+}
+template <int WAVES>
+__device__ __forceinline__ void set_row_scales(const Fusion& f, const float (&share)[SCALE_ROWS<WAVES>][SCALE_SHARES], float* r_s, int M, int K,
+                                               int wave, int lane) {
+  if (f.ss_in == nullptr) return;
+#pragma unroll
+  for (int i = 0; i < SCALE_ROWS<WAVES>; ++i) {
+    const int m = wave + i * WAVES;
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < SCALE_SHARES; ++j) sum += share[i][j];
+    if (m < M)
+      for (int t = lane + SCALE_SHARES * 64; t < f.tiles_in; t += 64) sum += f.ss_in[(size_t)m * f.tiles_in + t];
+    sum = wave_sum(sum);
+    if (m < M && lane == 0) r_s[m] = 1.0f / sqrtf(sum / (float)K + f.eps);
+  }
+}
+
+// What the wave that writes a tile adds to and multiplies with, asked for before the tile's weights: the residual's
+// entries and the next norm's weights of the lane's four outputs.
+__device__ __forceinline__ void read_residual(const Fusion& f, float (&ahead)[8], int col, int grp, int n0, int M, int N) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + grp * 4 + j;
+    ahead[4 + j] = 1.0f;
+    if (col < M && n < N) {
+      const size_t at = (size_t)col * N + n;
+      ahead[j] = f.residual_f32 ? reinterpret_cast<const float*>(f.residual)[at] : (float)reinterpret_cast<const bf16_t*>(f.residual)[at];
+      if (f.next_w) ahead[4 + j] = f.next_w_f32 ? reinterpret_cast<const float*>(f.next_w)[n] : (float)reinterpret_cast<const bf16_t*>(f.next_w)[n];
+    }
+  }
+}
+
+// A finished tile goes out: lane (col, grp) holds outputs n0 + 4 grp + (0..3) of row col of x. Plain: stored as they
+// are. With a residual stream (nhv_gemm_fusion.h): added to it in float, the sum kept there and, times the next
+// norm's weight and rounded, in sum_out, and the tile's share of the row's sum of squares (over its 16 outputs, the
+// lanes' shares added in a fixed order) in ss_out. `tile` and `tiles` count tiles of 16 outputs over all of N.
+// `ahead`: the residual's entries and the next norm's weights where the caller has read them already (read_residual), else null.
+template <bool FUSED, typename TOut>
+__device__ __forceinline__ void emit_tile(const Fusion& f, const float (&r)[4], TOut* __restrict__ y, int col, int grp, int n0,
+                                          int tile, int tiles, int M, int N, const float* ahead = nullptr) {
+  if (!FUSED || f.residual == nullptr) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + grp * 4 + j;
+      if (col < M && n < N) y[(size_t)col * N + n] = (TOut)r[j];
+    }
+    return;
+  }
+  float sq = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + grp * 4 + j;
+    if (col < M && n < N) {
+      const size_t at = (size_t)col * N + n;
+      float sum;
+      if (f.residual_f32) {
+        float* res = reinterpret_cast<float*>(f.residual);
+        sum = r[j] + (ahead ? ahead[j] : res[at]);
+        res[at] = sum;
+      } else {
+        bf16_t* res = reinterpret_cast<bf16_t*>(f.residual);
+        sum = r[j] + (ahead ? ahead[j] : (float)res[at]);
+        res[at] = (bf16_t)sum;
+      }
+      float weight = 1.0f;
+      if (ahead) weight = ahead[4 + j];
+      else if (f.next_w) weight = f.next_w_f32 ? reinterpret_cast<const float*>(f.next_w)[n] : (float)reinterpret_cast<const bf16_t*>(f.next_w)[n];
+      f.sum_out[at] = (bf16_t)(sum * weight);
+      sq += sum * sum;
+    }
+  }
+  sq += __shfl_xor(sq, 16, 64);
+  sq += __shfl_xor(sq, 32, 64);
+  if (grp == 0 && col < M) f.ss_out[(size_t)col * tiles + tile] = sq;
+}
+
 // NT: tiles of 16 rows of w per block; WAVES: waves that share the block's part of K; UNROLL: loads in
 // flight per wave and operand. A step is 32 columns of K (64 bytes of a row).
-template <int NT, int WAVES, int UNROLL, bool GLU, typename TOut>
+template <int NT, int WAVES, int UNROLL, bool GLU, bool FUSED, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                   const bf16_t* __restrict__ bias, TOut* __restrict__ y,
-                                                                  int M, int N, int K, int steps_per_wave) {
+                                                                  int M, int N, int K, int steps_per_wave, const Fusion f) {
   constexpr int NA = GLU ? 2 : 1;
   constexpr int TILES = NA * NT;
   static_assert(NT <= WAVES, "wave nt finishes tile nt");
   __shared__ float red[WAVES][TILES][4][64];
+  __shared__ float r_s[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int n0 = blockIdx.x * 16 * NT;
+  float share[SCALE_ROWS<WAVES>][SCALE_SHARES];
+  if constexpr (FUSED) ask_row_scales<WAVES>(f, share, M, wave, lane);
 
   const bf16_t* wrow[TILES];
   bool n_ok[NT];
@@ -88,6 +190,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_kernel(const bf16_t* 
 #pragma unroll
       for (int t = 0; t < TILES; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][t], b[u], acc[t], 0, 0, 0);
   }
+  if constexpr (FUSED) set_row_scales<WAVES>(f, share, r_s, M, K, wave, lane);
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
 #pragma unroll
@@ -108,16 +211,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_kernel(const bf16_t* 
       v[na][j] = sum;
     }
 
+  const float rs = (FUSED && f.ss_in) ? r_s[col] : 1.0f;           // the row's scale, where x is a sum whose norm is due
+  float out[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int n = n0 + nt * 16 + grp * 4 + j;           // the tile's row 4 grp + j is output n, its column is row col of x
-    if (col < M && n < N) {
-      float r = v[0][j];
-      if (bias) r += (float)bias[n];
-      if (GLU) r = r / (1.0f + expf(-r)) * v[NA - 1][j];
-      y[(size_t)col * N + n] = (TOut)r;
-    }
+    float r = v[0][j] * rs;
+    if (bias && n < N) r += (float)bias[n];
+    if (GLU) r = r / (1.0f + expf(-r)) * (v[NA - 1][j] * rs);
+    out[j] = r;
   }
+  emit_tile<FUSED, TOut>(f, out, y, col, grp, n0 + nt * 16, blockIdx.x * NT + nt, (N + 15) / 16, M, N);
 }
 
 typedef __attribute__((address_space(3))) void* lds_ptr;
@@ -129,10 +233,11 @@ typedef const __attribute__((address_space(1))) void* global_ptr;
 // The first weights of a block's first tile are asked for right after x and the wait before the first product is for
 // x alone (0.2 to 0.5 us less per call at every shape; asked for before x they made every shape slower, by 0.5 to
 // 3 us).
-template <int WAVES, int UNROLL, bool GLU, typename TOut>
+template <int WAVES, int UNROLL, bool GLU, bool FUSED, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                            const bf16_t* __restrict__ bias, TOut* __restrict__ y,
-                                                                           int M, int N, int K, int tiles, int steps_per_wave) {
+                                                                           int M, int N, int K, int tiles, int steps_per_wave,
+                                                                           const Fusion f) {
   constexpr int NA = GLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float(*red)[NA][4][64] = reinterpret_cast<float(*)[NA][4][64]>(lds_raw);      // [2 WAVES][NA][4][64]
@@ -140,6 +245,11 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
   const int pitch = K + 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
+  __shared__ float r_s[16];
+  // (the rows' scales are wanted when the first tile goes out: their shares are asked for first of all, and the
+  // barrier before the tile's sums are added up makes the scales visible)
+  float share[SCALE_ROWS<WAVES>][SCALE_SHARES];
+  if constexpr (FUSED) ask_row_scales<WAVES>(f, share, M, wave, lane);
   // x into LDS: a wave's load brings 64 consecutive 16-byte pieces of one row
   const int pieces_per_row = K / 8;
   const int loads_per_row = (pieces_per_row + 63) / 64;
@@ -177,6 +287,10 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
   for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x, parity ^= 1, turn = turn + 1 == WAVES ? 0 : turn + 1) {
     const int n0 = tile * 16;
     const bool n_ok = n0 + col < N;
+    // the wave that will write this tile asks for the residual's entries it adds to before the tile's weights
+    // (the gated product is never added to a residual stream)
+    float res_ahead[8] = {0.f, 0.f, 0.f, 0.f, 1.f, 1.f, 1.f, 1.f};
+    if constexpr (FUSED && !GLU) if (f.residual != nullptr && wave == turn) read_residual(f, res_ahead, col, grp, n0, M, N);
     const bf16_t* wrow[NA];
 #pragma unroll
     for (int na = 0; na < NA; ++na) wrow[na] = w + ((size_t)na * N + (n_ok ? n0 + col : 0)) * K;
@@ -205,6 +319,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
         for (int na = 0; na < NA; ++na) acc[na] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][na], b, acc[na], 0, 0, 0);
       }
     }
+    if constexpr (FUSED) if (tile == (int)blockIdx.x) set_row_scales<WAVES>(f, share, r_s, M, K, wave, lane);
     float(*my_red)[NA][4][64] = red + parity * WAVES;
 #pragma unroll
     for (int na = 0; na < NA; ++na)
@@ -222,27 +337,28 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
         for (int wv = 0; wv < WAVES; ++wv) sum += my_red[wv][na][j][lane];
         v[na][j] = sum;
       }
+    const float rs = (FUSED && f.ss_in) ? r_s[col] : 1.0f;         // the row's scale, where x is a sum whose norm is due
+    float out[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + grp * 4 + j;
-      if (col < M && n < N) {
-        float r = v[0][j];
-        if (bias) r += (float)bias[n];
-        if (GLU) r = r / (1.0f + expf(-r)) * v[NA - 1][j];
-        y[(size_t)col * N + n] = (TOut)r;
-      }
+      float r = v[0][j] * rs;
+      if (bias && n < N) r += (float)bias[n];
+      if (GLU) r = r / (1.0f + expf(-r)) * (v[NA - 1][j] * rs);
+      out[j] = r;
     }
+    emit_tile<FUSED && !GLU, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N, res_ahead);
   }
 }
 
 // Where all of x is too much for LDS: the same with one tile a block and x coming in `nchunks` pieces of
 // `chunk_steps` steps of 32 columns, one after the other; the sums run on over the pieces. (A kernel of its own:
 // as an option of the one above it cost that one 4 % of its speed.)
-template <int WAVES, int UNROLL, typename TOut>
+template <int WAVES, int UNROLL, bool FUSED, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                            const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                                            int M, int N, int K, int tiles, int nchunks,
-                                                                           int chunk_steps, int steps_per_wave) {
+                                                                           int chunk_steps, int steps_per_wave, const Fusion f) {
   constexpr int NA = 1;
   constexpr bool GLU = false;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -251,6 +367,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const b
   const int pitch = min(K, chunk_steps * 32) + 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
+  __shared__ float r_s[16];
+  float share[SCALE_ROWS<WAVES>][SCALE_SHARES];
+  if constexpr (FUSED) ask_row_scales<WAVES>(f, share, M, wave, lane);
   const int ksteps = (K + 31) / 32;
   const bool m_ok = col < M;
   const bf16_t* xrow_s = x_s + (m_ok ? col : 0) * pitch;
@@ -304,6 +423,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const b
         }
       }
     }
+    if constexpr (FUSED) if (tile == (int)blockIdx.x) set_row_scales<WAVES>(f, share, r_s, M, K, wave, lane);
     float(*my_red)[NA][4][64] = red + parity * WAVES;
 #pragma unroll
     for (int na = 0; na < NA; ++na)
@@ -321,16 +441,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const b
         for (int wv = 0; wv < WAVES; ++wv) sum += my_red[wv][na][j][lane];
         v[na][j] = sum;
       }
+    const float rs = (FUSED && f.ss_in) ? r_s[col] : 1.0f;         // the row's scale, where x is a sum whose norm is due
+    float out[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + grp * 4 + j;
-      if (col < M && n < N) {
-        float r = v[0][j];
-        if (bias) r += (float)bias[n];
-        if (GLU) r = r / (1.0f + expf(-r)) * v[NA - 1][j];
-        y[(size_t)col * N + n] = (TOut)r;
-      }
+      float r = v[0][j] * rs;
+      if (bias && n < N) r += (float)bias[n];
+      if (GLU) r = r / (1.0f + expf(-r)) * (v[NA - 1][j] * rs);
+      out[j] = r;
     }
+    emit_tile<FUSED, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N);
   }
 }
 
@@ -338,11 +459,12 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const b
 // steps of 32 columns; for every piece the block walks over all of its tiles, and a tile's sums over the pieces so
 // far wait in LDS (part_s, 1 KB a tile and matrix) for the next piece. The weights are still read once. The
 // wave that adds up a tile's sums is the same in every pass, so what it left in part_s it finds again itself.
-template <int WAVES, int UNROLL, bool GLU, typename TOut>
+template <int WAVES, int UNROLL, bool GLU, bool FUSED, typename TOut>
 __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_passes_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                            const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                                            int M, int N, int K, int tiles, int npasses,
-                                                                           int pass_steps, int steps_per_wave, int tiles_per_block) {
+                                                                           int pass_steps, int steps_per_wave, int tiles_per_block,
+                                                                           const Fusion f) {
   constexpr int NA = GLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float(*red)[NA][4][64] = reinterpret_cast<float(*)[NA][4][64]>(lds_raw);      // [2 WAVES][NA][4][64]
@@ -351,6 +473,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_passes_kernel(const b
   const int pitch = min(K, pass_steps * 32) + 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
+  __shared__ float r_s[16];
+  float share[SCALE_ROWS<WAVES>][SCALE_SHARES];
+  if constexpr (FUSED) ask_row_scales<WAVES>(f, share, M, wave, lane);
   const int ksteps = (K + 31) / 32;
   const bool m_ok = col < M;
   const bf16_t* xrow_s = x_s + (m_ok ? col : 0) * pitch;
@@ -403,6 +528,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_passes_kernel(const b
           for (int na = 0; na < NA; ++na) acc[na] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][na], b, acc[na], 0, 0, 0);
         }
       }
+      if constexpr (FUSED) if (p == 0 && ti == 0) set_row_scales<WAVES>(f, share, r_s, M, K, wave, lane);
       float(*my_red)[NA][4][64] = red + parity * WAVES;
 #pragma unroll
       for (int na = 0; na < NA; ++na)
@@ -427,21 +553,22 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_passes_kernel(const b
           for (int j = 0; j < 4; ++j) part_s[ti][na][j][lane] = v[na][j];
         continue;
       }
+      const float rs = (FUSED && f.ss_in) ? r_s[col] : 1.0f;       // the row's scale, where x is a sum whose norm is due
+      float out[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int n = n0 + grp * 4 + j;
-        if (col < M && n < N) {
-          float r = v[0][j];
-          if (bias) r += (float)bias[n];
-          if (GLU) r = r / (1.0f + expf(-r)) * v[NA - 1][j];
-          y[(size_t)col * N + n] = (TOut)r;
-        }
+        float r = v[0][j] * rs;
+        if (bias && n < N) r += (float)bias[n];
+        if (GLU) r = r / (1.0f + expf(-r)) * (v[NA - 1][j] * rs);
+        out[j] = r;
       }
+      emit_tile<FUSED, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N);
     }
   }
 }
 
-constexpr size_t LDS_BYTES = 160 * 1024;
+constexpr size_t LDS_BYTES = 160 * 1024 - 64;      // (64 bytes are the rows' scales, which every kernel keeps beside)
 
 // The resident kernel's shape: waves, loads in flight and blocks per compute unit, from the best variants measured
 // (same shapes as below), and in how many pieces x comes; waves == 0 when this kernel is not the one to take.
@@ -494,28 +621,28 @@ static ResidentPlan resident_plan(bool glu, int M, int N, int K) {
   return {waves, unroll, bpc < 2 ? 1 : 2, nchunks, chunk_steps, lds};
 }
 
-template <int WAVES, int UNROLL, bool GLU, bool PIECES, typename TOut>
+template <int WAVES, int UNROLL, bool GLU, bool PIECES, bool FUSED, typename TOut>
 static int launch_resident(const ResidentPlan& p, hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M,
-                           int N, int K) {
+                           int N, int K, const Fusion& f) {
   static_assert(!(GLU && PIECES), "x in pieces is not built for the gated kernel");
   const int steps_per_wave = 2 * ((p.chunk_steps + 2 * WAVES - 1) / (2 * WAVES));
   const int tiles = (N + 15) / 16;
   if constexpr (PIECES) {
-    auto kernel = gemm_fewrows_pieces_kernel<WAVES, UNROLL, TOut>;
+    auto kernel = gemm_fewrows_pieces_kernel<WAVES, UNROLL, FUSED, TOut>;
     // more than 64 KB of dynamic LDS has to be allowed once per kernel (and per process)
     static const hipError_t allowed =
         hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
     if (allowed != hipSuccess) return nhv_fail("few-rows gemm: %s", hipGetErrorString(allowed));
     hipLaunchKernelGGL(kernel, dim3(tiles), dim3(64 * WAVES), p.lds, s, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias,
-                       (TOut*)y, M, N, K, tiles, p.nchunks, p.chunk_steps, steps_per_wave);
+                       (TOut*)y, M, N, K, tiles, p.nchunks, p.chunk_steps, steps_per_wave, f);
   } else {
-    auto kernel = gemm_fewrows_resident_kernel<WAVES, UNROLL, GLU, TOut>;
+    auto kernel = gemm_fewrows_resident_kernel<WAVES, UNROLL, GLU, FUSED, TOut>;
     static const hipError_t allowed =
         hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
     if (allowed != hipSuccess) return nhv_fail("few-rows gemm: %s", hipGetErrorString(allowed));
     const int grid = tiles < 256 * p.blocks_per_cu ? tiles : 256 * p.blocks_per_cu;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * WAVES), p.lds, s, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias,
-                       (TOut*)y, M, N, K, tiles, steps_per_wave);
+                       (TOut*)y, M, N, K, tiles, steps_per_wave, f);
   }
   return 0;
 }
@@ -543,17 +670,17 @@ static PassesPlan passes_plan(bool glu, int M, int N, int K) {
   return {0, 0, 0, 0, 0, 0, 0};
 }
 
-template <int WAVES, int UNROLL, bool GLU, typename TOut>
+template <int WAVES, int UNROLL, bool GLU, bool FUSED, typename TOut>
 static int launch_passes(const PassesPlan& p, hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M, int N,
-                         int K) {
-  auto kernel = gemm_fewrows_passes_kernel<WAVES, UNROLL, GLU, TOut>;
+                         int K, const Fusion& f) {
+  auto kernel = gemm_fewrows_passes_kernel<WAVES, UNROLL, GLU, FUSED, TOut>;
   // more than 64 KB of dynamic LDS has to be allowed once per kernel (and per process)
   static const hipError_t allowed =
       hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
   if (allowed != hipSuccess) return nhv_fail("few-rows gemm: %s", hipGetErrorString(allowed));
   const int steps_per_wave = 2 * ((p.pass_steps + 2 * WAVES - 1) / (2 * WAVES));
   hipLaunchKernelGGL(kernel, dim3(p.grid), dim3(64 * WAVES), p.lds, s, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias,
-                     (TOut*)y, M, N, K, (N + 15) / 16, p.npasses, p.pass_steps, steps_per_wave, p.tiles_per_block);
+                     (TOut*)y, M, N, K, (N + 15) / 16, p.npasses, p.pass_steps, steps_per_wave, p.tiles_per_block, f);
   return 0;
 }
 
@@ -587,16 +714,19 @@ static Plan plan(bool glu, int M, int N, int K) {
 
 template <int NT, int WAVES, int UNROLL, bool GLU>
 static void launch(hipStream_t s, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
-                   int out_dtype) {
+                   int out_dtype, bool fused, const Fusion& f) {
   const int ksteps = (K + 31) / 32;
   const int steps_per_wave = 2 * ((ksteps + 2 * WAVES - 1) / (2 * WAVES));     // even: whole cache lines of 128 bytes
   const unsigned blocks = (unsigned)((N + 16 * NT - 1) / (16 * NT));
-  if (out_dtype == NHV_BF16)
-    hipLaunchKernelGGL((gemm_fewrows_kernel<NT, WAVES, UNROLL, GLU, bf16_t>), dim3(blocks), dim3(64 * WAVES), 0, s,
-                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, M, N, K, steps_per_wave);
+  if (fused)
+    hipLaunchKernelGGL((gemm_fewrows_kernel<NT, WAVES, UNROLL, GLU, true, bf16_t>), dim3(blocks), dim3(64 * WAVES), 0, s,
+                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, M, N, K, steps_per_wave, f);
+  else if (out_dtype == NHV_BF16)
+    hipLaunchKernelGGL((gemm_fewrows_kernel<NT, WAVES, UNROLL, GLU, false, bf16_t>), dim3(blocks), dim3(64 * WAVES), 0, s,
+                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, M, N, K, steps_per_wave, f);
   else
-    hipLaunchKernelGGL((gemm_fewrows_kernel<NT, WAVES, UNROLL, GLU, float>), dim3(blocks), dim3(64 * WAVES), 0, s,
-                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (float*)y, M, N, K, steps_per_wave);
+    hipLaunchKernelGGL((gemm_fewrows_kernel<NT, WAVES, UNROLL, GLU, false, float>), dim3(blocks), dim3(64 * WAVES), 0, s,
+                       (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (float*)y, M, N, K, steps_per_wave, f);
 }
 
 }  // namespace fewrows
@@ -604,13 +734,17 @@ static void launch(hipStream_t s, const void* x, const void* w, const void* bias
 // The caller has checked sizes, alignment and types (1 <= M <= 16, K a multiple of 8). Returns 0, or 1 with the
 // error message set.
 int nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
-                            int out_dtype, hipStream_t s) {
+                            int out_dtype, hipStream_t s, const NhvGemmFusion& f) {
   using namespace fewrows;
+  // a product that takes over work of its neighbours is a kernel of its own kind (more registers): bfloat16 results only
+  const bool fused = f.residual != nullptr || f.ss_in != nullptr;
+  if (fused && out_dtype != NHV_BF16) return nhv_fail("few-rows gemm: a product that takes over its neighbours' work gives bfloat16");
   const ResidentPlan rp = resident_plan(glu, M, N, K);
 #define NHV_RESIDENT_CASE(WV_, UN_, GLU_, PIECES_)                                                                     \
   if (rp.waves == WV_ && rp.unroll == UN_ && glu == GLU_ && (rp.nchunks > 1) == PIECES_)                              \
-    return out_dtype == NHV_BF16 ? launch_resident<WV_, UN_, GLU_, PIECES_, bf16_t>(rp, s, x, w, bias, y, M, N, K)    \
-                                 : launch_resident<WV_, UN_, GLU_, PIECES_, float>(rp, s, x, w, bias, y, M, N, K);
+    return fused                   ? launch_resident<WV_, UN_, GLU_, PIECES_, true, bf16_t>(rp, s, x, w, bias, y, M, N, K, f)  \
+           : out_dtype == NHV_BF16 ? launch_resident<WV_, UN_, GLU_, PIECES_, false, bf16_t>(rp, s, x, w, bias, y, M, N, K, f) \
+                                   : launch_resident<WV_, UN_, GLU_, PIECES_, false, float>(rp, s, x, w, bias, y, M, N, K, f);
   NHV_RESIDENT_CASE(8, 2, true, false)
   NHV_RESIDENT_CASE(4, 8, true, false)
   NHV_RESIDENT_CASE(16, 2, false, false)
@@ -627,8 +761,9 @@ int nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* 
     const PassesPlan pp = passes_plan(glu, M, N, K);
 #define NHV_PASSES_CASE(WV_, UN_, GLU_)                                                                  \
   if (pp.npasses == 2 && pp.waves == WV_ && pp.unroll == UN_ && glu == GLU_)                             \
-    return out_dtype == NHV_BF16 ? launch_passes<WV_, UN_, GLU_, bf16_t>(pp, s, x, w, bias, y, M, N, K)  \
-                                 : launch_passes<WV_, UN_, GLU_, float>(pp, s, x, w, bias, y, M, N, K);
+    return fused                   ? launch_passes<WV_, UN_, GLU_, true, bf16_t>(pp, s, x, w, bias, y, M, N, K, f)  \
+           : out_dtype == NHV_BF16 ? launch_passes<WV_, UN_, GLU_, false, bf16_t>(pp, s, x, w, bias, y, M, N, K, f) \
+                                   : launch_passes<WV_, UN_, GLU_, false, float>(pp, s, x, w, bias, y, M, N, K, f);
     NHV_PASSES_CASE(8, 2, true)
     NHV_PASSES_CASE(4, 8, true)
     NHV_PASSES_CASE(16, 2, false)
@@ -638,7 +773,7 @@ int nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* 
   const Plan p = plan(glu, M, N, K);
 #define NHV_FEWROWS_CASE(NT_, WV_, UN_, GLU_)                                              \
   if (p.nt == NT_ && p.waves == WV_ && p.unroll == UN_ && glu == GLU_) {                   \
-    launch<NT_, WV_, UN_, GLU_>(s, x, w, bias, y, M, N, K, out_dtype);                     \
+    launch<NT_, WV_, UN_, GLU_>(s, x, w, bias, y, M, N, K, out_dtype, fused, f);           \
     return 0;                                                                              \
   }
   NHV_FEWROWS_CASE(1, 8, 8, false)

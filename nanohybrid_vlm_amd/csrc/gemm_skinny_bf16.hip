@@ -2,12 +2,14 @@
 // matrix products of a decoding step, and the kernel for 17 to 64 rows. Up to 16 rows go to the kernel in
 // gemm_fewrows_bf16.hip.
 #include "nhv_common.h"
+#include "nhv_gemm_fusion.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 int nhv_gemm_fewrows_launch(bool glu, const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
-                            int out_dtype, hipStream_t s);
+                            int out_dtype, hipStream_t s, const NhvGemmFusion& f);
+static const NhvGemmFusion NO_FUSION = {};
 
 __device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x8 sk_zero8() {
@@ -158,7 +160,7 @@ extern "C" int nhv_gemm_skinny_bf16(const void* x, const void* w, const void* bi
     NHV_LAUNCH_CHECK("gemm_mid_bf16");
     return 0;
   }
-  if (nhv_gemm_fewrows_launch(false, x, w, bias, y, M, N, K, out_dtype, s)) return 1;
+  if (nhv_gemm_fewrows_launch(false, x, w, bias, y, M, N, K, out_dtype, s, NO_FUSION)) return 1;
   NHV_LAUNCH_CHECK("gemm_fewrows_bf16");
   return 0;
 }
@@ -173,7 +175,46 @@ extern "C" int nhv_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, i
     NHV_LAUNCH_CHECK("gemm_mid_glu_bf16");
     return 0;
   }
-  if (nhv_gemm_fewrows_launch(true, x, w, nullptr, y, M, N, K, out_dtype, s)) return 1;
+  if (nhv_gemm_fewrows_launch(true, x, w, nullptr, y, M, N, K, out_dtype, s, NO_FUSION)) return 1;
   NHV_LAUNCH_CHECK("gemm_fewrows_glu_bf16");
+  return 0;
+}
+
+// ---- products of up to 16 rows that take over the kernels around them (nhv_gemm_fusion.h) ----
+// y = r . (x . w^T) (+ bias), or with glu silu(r . (x . w[0:N]^T)) * (r . (x . w[N:2N]^T)), for 1 <= M <= 16 rows in
+// bfloat16. With ss_in: x is a sum (times its norm's weight) whose rows still lack their scales: r per row from ss_in
+// [M, tiles_in] (the tiles' shares of the row's sum of squares over its K entries) and eps; without: r = 1.
+// With residual: the product is not stored; it is added to residual [M, N] (float or bfloat16, rewritten), the sum
+// times next_w [N] (if given), rounded, goes to sum_out [M, N] (bfloat16) and the tiles' shares of its rows' sums of
+// squares to ss_out [M, (N + 15) / 16]; y is then not touched (may be null). Not with glu.
+extern "C" int nhv_gemm_fewrows_fused_bf16(const void* x, const void* ss_in, int tiles_in, float eps, const void* w,
+                                           const void* bias, void* y, int M, int N, int K, int out_dtype, int glu,
+                                           void* residual, int residual_dtype, void* sum_out, void* ss_out,
+                                           const void* next_w, int next_w_dtype, void* stream) {
+  if (sk_check("fused few-rows gemm", x, w, M, N, K, out_dtype)) return 1;
+  NHV_REQUIRE(M <= 16, "fused few-rows gemm: %d rows are beyond this kernel's limit of 16", M);
+  NhvGemmFusion f = {};
+  if (ss_in) {
+    NHV_REQUIRE(tiles_in > 0 && eps > 0.f, "fused few-rows gemm: the rows' scales need the tiles' count and eps");
+    f.ss_in = (const float*)ss_in;
+    f.tiles_in = tiles_in;
+    f.eps = eps;
+  }
+  if (residual) {
+    NHV_REQUIRE(!glu, "fused few-rows gemm: the gated product is not added to a residual");
+    NHV_REQUIRE(sum_out && ss_out, "fused few-rows gemm: the sum and its squares need a place");
+    NHV_REQUIRE(residual_dtype == NHV_F32 || residual_dtype == NHV_BF16, "fused few-rows gemm: residual of unknown type %d", residual_dtype);
+    NHV_REQUIRE(!next_w || next_w_dtype == NHV_F32 || next_w_dtype == NHV_BF16, "fused few-rows gemm: norm weight of unknown type %d", next_w_dtype);
+    f.residual = residual;
+    f.residual_f32 = residual_dtype == NHV_F32;
+    f.sum_out = (bf16_t*)sum_out;
+    f.ss_out = (float*)ss_out;
+    f.next_w = next_w;
+    f.next_w_f32 = next_w_dtype == NHV_F32;
+  } else {
+    NHV_REQUIRE(y != nullptr, "fused few-rows gemm: no place for the result");
+  }
+  if (nhv_gemm_fewrows_launch(glu != 0, x, w, glu ? nullptr : bias, y, M, N, K, out_dtype, (hipStream_t)stream, f)) return 1;
+  NHV_LAUNCH_CHECK("gemm_fewrows_fused_bf16");
   return 0;
 }

@@ -142,7 +142,7 @@ class LLM:
         if built_model is None and not os.path.isdir(model):
             raise FileNotFoundError(f"model folder '{model}' does not exist")
         arch, typed, built = built_model if built_model is not None else (None, None, None)
-        self._set_up_gemm_choices(cfg)
+        gemm_table, measure_gemms = self._gemm_choices_of(cfg)
         self.runner = ModelRunner(
             model, dtype=cfg.dtype, device=cfg.device, page_size=cfg.kvcache_block_size,
             num_pages=None if cfg.num_kvcache_blocks == -1 else cfg.num_kvcache_blocks,
@@ -150,7 +150,8 @@ class LLM:
             gpu_memory_utilization=cfg.gpu_memory_utilization, max_num_batched_tokens=cfg.max_num_batched_tokens,
             model=built, arch=arch, cfg=typed, use_graphs=not cfg.enforce_eager, max_model_len=cfg.max_model_len,
             share_prefixes=cfg.enable_prefix_cache, max_graph_batch=cfg.max_graph_batch, max_graph_tokens=cfg.max_graph_tokens,
-            residual_float32=cfg.residual_dtype == "float32", poison_freed_pages=poison_freed_pages)
+            residual_float32=cfg.residual_dtype == "float32", poison_freed_pages=poison_freed_pages,
+            gemm_table=gemm_table, measure_gemms=measure_gemms, fuse_norms=cfg.fuse_norms)
         cfg.num_kvcache_blocks = self.runner.num_pages
         # max_model_len is capped by the model's positions (nanovllm/config.py:420-423); both, and the token that
         # ends a request, are facts of the built model (no field of an architecture's configuration is read here)
@@ -179,27 +180,32 @@ class LLM:
 
     # ------------------------------------------------------------------ how matrix products are done
     @staticmethod
-    def _set_up_gemm_choices(cfg: EngineConfig) -> None:
-        """Tells the kernel library whether it may time matrix products, and gives it a table of choices made by an
-        earlier run. With a table (or with measuring off) the same kernels run in every process: logits are the same
-        bit for bit from start to start, and no step pays for a measurement."""
+    def _gemm_choices_of(cfg: EngineConfig) -> tuple[dict | None, bool]:
+        """(this engine's table of choices, whether shapes it lacks may be timed). With a table read from a file, or
+        with measuring off, the same kernels run in every process: logits are the same bit for bit from start to
+        start, and no step pays for a measurement. An engine with a file of choices, or with measuring off, has a
+        table of its own; any other shares the process-wide table, in which a shape is timed once for all engines."""
         import json
         from ..native import ops
         backend = ops.backend()
-        if not hasattr(backend, "load_choices"):
-            return                                     # (a stand-in for the kernels has nothing to choose)
-        backend.measuring_allowed = bool(cfg.measure_gemms)
+        if not hasattr(backend, "parse_choices"):
+            return None, False                         # (a stand-in for the kernels has nothing to choose)
         if cfg.gemm_choices and os.path.isfile(cfg.gemm_choices):
             with open(cfg.gemm_choices) as f:
-                backend.load_choices(json.load(f))
-            backend.measuring_allowed = False
+                return backend.parse_choices(json.load(f)), False
+        if cfg.gemm_choices or not cfg.measure_gemms:
+            return {}, bool(cfg.measure_gemms)
+        return None, True
 
     def gemm_choices(self) -> dict:
-        """How each shape of matrix product met so far is done ("M,N,K,float result,gated" -> -1 own kernel, -2 the
-        rule, or a library algorithm's number)."""
+        """How each shape of matrix product that this engine's table holds is done ("M,N,K,float result,gated" ->
+        -1 own kernel, -2 the rule, or a library algorithm's number)."""
         from ..native import ops
         backend = ops.backend()
-        return backend.choices_table() if hasattr(backend, "choices_table") else {}
+        if not hasattr(backend, "choices_table"):
+            return {}
+        table = self.runner.gemm_table
+        return backend.choices_table(backend.shared_chosen if table is None else table)
 
     def save_gemm_choices(self, path: str | None = None) -> str:
         """Writes the choices made so far to ``path`` (default: the engine option ``gemm_choices``); a later run

@@ -52,9 +52,14 @@ class ModelRunner:
                  num_pages: int | None = None, num_state_slots: int = 512, gpu_memory_utilization: float = 0.9,
                  max_num_batched_tokens: int = 16384, model=None, arch=None, cfg=None, use_graphs: bool = False,
                  max_model_len: int | None = None, max_graph_batch: int = 64, poison_freed_pages: bool = False,
-                 share_prefixes: bool = False, residual_float32: bool = True, max_graph_tokens: int = 256):
+                 share_prefixes: bool = False, residual_float32: bool = True, max_graph_tokens: int = 256,
+                 gemm_table: dict | None = None, measure_gemms: bool = True, fuse_norms: bool = True):
         """``model``/``arch``/``cfg`` may be given ready-made (weights already bound)
-        instead of being read from ``model_dir``."""
+        instead of being read from ``model_dir``.
+        ``gemm_table``: this engine's own table of how each shape of bfloat16 matrix product is done (None: the
+        process-wide table, in which a shape is timed once for all engines); ``measure_gemms``: whether shapes that
+        the table lacks may be timed. Both are put in force whenever this runner steps, so engines of one process
+        do not change each other's products."""
         if dtype not in _TORCH_DTYPES:
             raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
         self.dtype = _TORCH_DTYPES[dtype]
@@ -81,6 +86,10 @@ class ModelRunner:
             raise ValueError("a freed page keeps its content for later requests when prefixes are shared; "
                              "poison_freed_pages would destroy it")
         self.share_prefixes = share_prefixes
+        self.gemm_table, self.measure_gemms = gemm_table, bool(measure_gemms)
+        # bfloat16 products of up to 16 rows may make the residual addition that follows them and the norm that comes
+        # before them in their own kernels (two kernels fewer a layer in a decoding step)
+        self.fuse_norms = bool(fuse_norms)
         self._pinned = None
         self._pinned_free = None
         # a debugging aid: pages that are given back are filled with NaN, so that a read of a page that a
@@ -256,7 +265,7 @@ class ModelRunner:
                 # and the matrix products of every new size of step are timed once: a sweep of the caches and a workspace
                 from ..native import ops
                 backend = ops.backend()
-                if getattr(backend, "measuring_allowed", False):
+                if self.measure_gemms and hasattr(backend, "library_workspace"):
                     own += (512 << 20) + 2 * getattr(backend, "library_workspace", 0)
         finally:
             # the probe's cache, its graphs and whatever the allocator kept go back to the device
@@ -542,6 +551,7 @@ class ModelRunner:
         """Runs the batch and returns float32 logits [wanted, vocab] in the order of the
         entries and of each entry's ``want`` (None if nothing is wanted). With ``keep=False`` the result may be
         memory that the next step overwrites (a caller that samples at once saves the copy)."""
+        self._use_own_choices()
         # (a recorded step of a model with one position axis has no array for positions of an entry's own)
         recorded = self.use_graphs and (self.position_axes > 1 or all(e.positions is None for e in entries))
         if recorded and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries):
@@ -569,6 +579,15 @@ class ModelRunner:
         for e, n in zip(entries, new_lens):
             self._poison(self.cache.commit(e.request_id, n, e.tokens))
         return logits
+
+    def _use_own_choices(self) -> None:
+        """This engine's table of matrix-product choices, and its leave to time, are the ones in force from here on."""
+        if self.device.type == "cuda":
+            from ..native import ops
+            backend = ops.backend()
+            if hasattr(backend, "use_choices"):
+                backend.use_choices(self.gemm_table, self.measure_gemms)
+                backend.fuse_norms = self.fuse_norms
 
     def _poison(self, given_back: list[list[int]]) -> None:
         if not self.poison_freed_pages or not any(given_back):
@@ -669,6 +688,7 @@ class ModelRunner:
         ``can_step_ahead``. The GPU goes from one step into the next while the host still waits for the tokens,
         finishes the step before and plans: between two steps that the host issues in turn the GPU waits 0.1 to
         0.3 ms. Returns what ``logits_ahead`` and ``undo_ahead`` need."""
+        self._use_own_choices()
         entries = [StepEntry(r, [0], [0]) for r in request_ids]
         bucket = next(b for b in self.graph_buckets if b >= len(entries))
         g = self._graphs[bucket]
@@ -762,9 +782,16 @@ class ModelRunner:
                     t[state_slots] = rows[name]
 
         try:
-            # warm-up; it writes the same cache slots as every replay will
-            eager = self.model.logits(self.model.forward(ctx)).clone()
-            torch.cuda.synchronize()
+            # warm-up; it writes the same cache slots as every replay will. A run in which a product's shape was
+            # measured is run again: how one product is done can depend on what was found out about a later one, and
+            # the recorded step is compared with an eager one that was done the same way throughout
+            for _ in range(3):
+                known = len(getattr(backend, "chosen", ()))
+                eager = self.model.logits(self.model.forward(ctx)).clone()
+                torch.cuda.synchronize()
+                if len(getattr(backend, "chosen", ())) == known:
+                    break
+                put_state_back()
             graph = torch.cuda.CUDAGraph()
             try:
                 if self._graph_pool is None:

@@ -107,6 +107,7 @@ class NativeBackend:
     measure_linears = False       # True: a product of few rows and a shape not seen before is timed in every way there is (see _choose)
     measure_many_rows = True      # a product of more than library_rows rows is timed in the third step that meets its shape
     measuring_allowed = True      # False: nothing is ever timed; a shape follows the table that was loaded, or the rule
+    fuse_norms = True             # products of up to few_rows rows may take over the residual addition and the norm around them (see Summed, Normed)
     step_number = 0               # counted by the engine, one per eager step
 
     def __init__(self):
@@ -115,9 +116,14 @@ class NativeBackend:
         self.lib = library.load_library("nhv_core", CORE_SOURCES)
         self.lib.nhv_last_error.restype = ctypes.c_char_p
         self._attention_libs: dict[int, ctypes.CDLL] = {}
-        self.chosen: dict[tuple, int] = {}                  # (M, N, K, float result, gated) of a product -> OWN or a library algorithm, measured
+        # (M, N, K, float result, gated) of a product -> OWN, RULE or a library algorithm, measured. ``chosen`` is the
+        # table in force: the process-wide one that engines share by default (a shape is timed once per process), or
+        # the table of the engine that runs now (see ``use_choices``)
+        self.shared_chosen: dict[tuple, int] = {}
+        self.chosen: dict[tuple, int] = self.shared_chosen
         self._blas = None
         self._plans: dict[tuple, tuple[int, int]] = {}
+        self.times: dict[tuple, tuple[float, float]] = {}   # measured shape -> (ms of the own kernel, ms of the library's best), cold
         self._met: dict[tuple, tuple[int, int]] = {}        # shape of many rows -> (steps that met it, the last of them)
         self._workspace = None
         self._sweep = None                                  # scratch memory whose reading empties the caches before a measurement
@@ -363,6 +369,9 @@ class NativeBackend:
         # cost inside a step is the harder one to measure alone)
         if incumbent_time is not None and how != incumbent and best[0][0] >= (0.90 if gated else 0.95) * incumbent_time:
             how = incumbent
+        library_times = [t for t, h in best + once if h >= 0]
+        if incumbent_time is not None and library_times:
+            self.times[(M, N, K, float_result, gated)] = (incumbent_time, min(library_times))
         if os.environ.get("NHV_SHOW_MEASUREMENTS"):
             name = {OWN: "own", RULE: "torch.mm"}
             first_guess = next((t for t, h in once if h == 0), float("nan"))
@@ -373,14 +382,16 @@ class NativeBackend:
         return how
 
     # -- the table of choices, so that a process can run by what another one measured --
-    def choices_table(self) -> dict[str, int]:
-        """What has been chosen so far, by shape: "M,N,K,float result,gated" -> -1 (own kernel), -2 (the rule:
-        ``torch.mm``) or the number of a library algorithm."""
-        return {",".join(str(int(v)) for v in key): how for key, how in sorted(self.chosen.items())}
+    def choices_table(self, chosen: dict | None = None) -> dict[str, int]:
+        """A table of choices (default: the one in force), by shape: "M,N,K,float result,gated" -> -1 (own kernel),
+        -2 (the rule: ``torch.mm``) or the number of a library algorithm."""
+        chosen = self.chosen if chosen is None else chosen
+        return {",".join(str(int(v)) for v in key): how for key, how in sorted(chosen.items())}
 
-    def load_choices(self, table: dict[str, int]) -> None:
-        """Takes a table as ``choices_table`` gives it. An entry that names a library algorithm is checked against
-        the library's list for the shape when it is first used (``nhv_library_gemm`` refuses a number beyond it)."""
+    def parse_choices(self, table: dict[str, int]) -> dict[tuple, int]:
+        """A table as ``choices_table`` gives it, as a table of this backend's own kind. Every entry is checked
+        now: its shape's form, and a library algorithm's number against the library's list for that shape."""
+        out = {}
         for text, how in table.items():
             parts = text.split(",")
             if len(parts) != 5:
@@ -388,7 +399,17 @@ class NativeBackend:
             M, N, K, f, g = (int(v) for v in parts)
             if not isinstance(how, int) or how < RULE:
                 raise KernelError(f"choice {how!r} for the product '{text}' is neither -1, -2 nor an algorithm's number")
-            self.chosen[(M, N, K, bool(f), bool(g))] = how
+            if how >= 0:
+                _, count = self._library_plan(M, N, K, bool(f) and not bool(g))
+                if how >= count:
+                    raise KernelError(f"choice {how} for the product '{text}': the library names {count} algorithms for this shape")
+            out[(M, N, K, bool(f), bool(g))] = how
+        return out
+
+    def use_choices(self, table: dict | None, measuring: bool) -> None:
+        """Puts an engine's table in force (None: the process-wide one) and says whether shapes that it lacks may be timed."""
+        self.chosen = self.shared_chosen if table is None else table
+        self.measuring_allowed = bool(measuring)
 
     def end_measurements(self) -> None:
         """Gives the scratch memory of the measurements back (what was measured stays known)."""
@@ -423,6 +444,76 @@ class NativeBackend:
                 return None
         self._call("nhv_gemm_generic", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K, dtype_code(x),
                    dtype_code(out), _stream())
+
+    norm_kernel_ms = 0.003        # what a norm's own kernel costs in a decoding step, about
+
+    def _measured(self, x, w, gated: bool):
+        """(the choice for this shape, (ms of the own kernel, ms of the library's best) or None); the shape is
+        measured here if it is due, as ``linear`` would have it measured."""
+        M, K = x.shape
+        key = (M, w.shape[0], K, False, gated)
+        how = self.chosen.get(key)
+        if how is None and self.measure_linears and self.measuring_allowed and not torch.cuda.is_current_stream_capturing():
+            scratch = torch.empty((M, w.shape[0] // 2 if gated else w.shape[0]), dtype=x.dtype, device=x.device)
+            how = self._choose(x, w, scratch, gated=gated)
+        return how, self.times.get(key)
+
+    def fusion_pays(self, x, w, gated: bool = False) -> bool:
+        """For a product whose rows come as a sum that still lacks its norm's scales: whether the own kernel, which
+        scales its sums itself, beats what this shape is otherwise done by. Where a measurement chose a library
+        algorithm for the shape, that algorithm and a kernel that scales the rows first have to be slower together
+        than the own kernel alone."""
+        if self.own_kernels_only:
+            return True
+        how, times = self._measured(x, w, gated)
+        if how is None or how < 0:
+            return True
+        if times is None:
+            return False                                     # (a choice from a table: followed as it stands)
+        own, library = times
+        return own <= library + self.norm_kernel_ms
+
+    def addition_pays(self, x, w, reader_w=None, reader_gated: bool = False) -> bool:
+        """For a product whose result is about to be added to the residual stream and normed: whether the own
+        kernel, which makes the addition itself, is the one to take. That saves the norm's kernel only if the product
+        that reads the norm (``reader_w``, of the same rows) scales its rows itself, so the two are priced together:
+        own kernels for both, against each one's best way and the norm's kernel between them. Without times for both
+        shapes the own kernel is taken where it is this shape's choice anyway."""
+        if self.own_kernels_only:
+            return True
+        how, times = self._measured(x, w, False)
+        if how is None or how < 0:
+            return True
+        if times is None or reader_w is None:
+            return False
+        reader_how = self.chosen.get((x.shape[0], reader_w.shape[0], reader_w.shape[1], False, reader_gated))
+        reader_times = self.times.get((x.shape[0], reader_w.shape[0], reader_w.shape[1], False, reader_gated))
+        if reader_how is None:
+            return False                                     # (the reader's shape is not measured yet: next time)
+        if reader_times is None:
+            if reader_how >= 0:
+                return False
+            reader_times = (0.0, 0.0)                        # the own kernel is the reader's way whatever is fused
+        own, library = times
+        reader_own, reader_library = reader_times
+        return own + reader_own <= min(own, library) + self.norm_kernel_ms + min(reader_own, reader_library)
+
+    def fused_linear(self, x, w, bias, out, gated=False, row_scales=None, residual=None, sum_out=None, ss_out=None, next_w=None):
+        """The own few-rows product with what it may take over. ``row_scales`` = (squares [M, tiles], eps): x is a
+        sum whose rows still lack their norm's scales, which are applied to the finished sums. ``residual``: the
+        result is added to it (in place); ``sum_out`` gets the sum times ``next_w`` (the next norm's weight), rounded,
+        and ``ss_out`` the tiles' shares of the rows' sums of squares (``out`` is then not written)."""
+        M, K = x.shape
+        N = w.shape[0] // 2 if gated else w.shape[0]
+        ss, eps = row_scales if row_scales is not None else (None, 0.0)
+        self._call("nhv_gemm_fewrows_fused_bf16", _ptr(x), _ptr(ss), 0 if ss is None else ss.shape[1], ctypes.c_float(eps),
+                   _ptr(w), _ptr(bias), _ptr(out), M, N, K, BF16 if out is None else dtype_code(out), int(gated),
+                   _ptr(residual), F32 if residual is None else dtype_code(residual), _ptr(sum_out), _ptr(ss_out),
+                   _ptr(next_w), F32 if next_w is None else dtype_code(next_w), _stream())
+
+    def scale_rows(self, x, squares, eps, out):
+        self._call("nhv_scale_rows", _ptr(x), _ptr(squares), squares.shape[1], ctypes.c_float(eps), _ptr(out), x.shape[0],
+                   x.shape[1], _stream())
 
     def gated_linear(self, x, w, out) -> bool:
         """silu(x Wg^T) * (x Wu^T) in one kernel, if this batch is one for the few-rows kernel; else False."""
@@ -535,6 +626,86 @@ def set_backend(obj) -> None:
     without a GPU put a stand-in here; the engine itself never does)."""
     global _backend
     _backend = obj
+
+
+# ------------------------------------------------------------------ work that a product takes over from its neighbours
+@dataclass
+class AddTo:
+    """What a part is handed in place of nothing when its result is about to be added to the residual stream and
+    normed: the stream, the weight and eps of the norm that follows, and (if known) the first product of the part
+    that reads that norm, as (weight, gated): whether making the addition in the product's kernel pays depends on
+    whether that reader scales its rows itself."""
+
+    residual: torch.Tensor
+    norm_weight: torch.Tensor
+    eps: float
+    reader: tuple | None = None
+
+
+@dataclass
+class Summed:
+    """What ``linear(..., add_to=AddTo(...))`` returns where the product's own kernel has made the addition: the
+    residual stream holds the sum already. ``weighted`` is the sum times the weight of the norm that follows, in
+    the rows' element type; ``squares`` [rows, tiles] holds every tile's share of each row's sum of squares. What the
+    norm still has to do is scale the rows: a product that reads ``Normed(summed)`` does that itself."""
+
+    weighted: torch.Tensor
+    squares: torch.Tensor
+    residual: torch.Tensor
+    norm_weight: torch.Tensor
+    eps: float
+
+    @property
+    def shape(self):
+        return self.weighted.shape
+
+
+@dataclass
+class Normed:
+    """The norm of a ``Summed`` with the scaling of its rows left to the product that reads it (``linear``,
+    ``gated_linear``: a product is linear in its rows, so it scales its own sums). ``tensor()`` is the norm as a
+    tensor, for any other reader (one small kernel)."""
+
+    summed: Summed
+
+    @property
+    def shape(self):
+        return self.summed.weighted.shape
+
+    def tensor(self) -> torch.Tensor:
+        s = self.summed
+        out = torch.empty_like(s.weighted)
+        backend().scale_rows(s.weighted, s.squares, float(s.eps), out)
+        return out
+
+
+def dense(x):
+    """``x`` as a tensor, whatever work was left undone in it."""
+    if isinstance(x, Normed):
+        return x.tensor()
+    if isinstance(x, Summed):
+        raise KernelError("a sum that was made for a norm (ops.Summed) goes through that norm, not anywhere else")
+    return x
+
+
+def _may_fuse(x: torch.Tensor, w: torch.Tensor) -> bool:
+    b = backend()
+    return (getattr(b, "fuse_norms", False) and hasattr(b, "fused_linear") and x.dtype == torch.bfloat16
+            and x.shape[0] <= getattr(b, "few_rows", 0) and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
+def _fusion_pays(x: torch.Tensor, w: torch.Tensor, gated: bool) -> bool:
+    pays = getattr(backend(), "fusion_pays", None)
+    return True if pays is None else pays(x, w, gated=gated)
+
+
+def _addition_pays(x: torch.Tensor, w: torch.Tensor, add_to: AddTo) -> bool:
+    pays = getattr(backend(), "addition_pays", None)
+    if pays is None:
+        return True
+    reader_w, reader_gated = add_to.reader if add_to.reader is not None else (None, False)
+    return pays(x, w, reader_w, reader_gated)
 
 
 # ------------------------------------------------------------------ checked entry points
@@ -688,9 +859,19 @@ def paged_attention(q, k_cache, v_cache, batch: AttentionBatch, block_tables, sc
     return out
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, out_dtype=None) -> torch.Tensor:
+def linear(x, w: torch.Tensor, bias: torch.Tensor | None = None, out_dtype=None, add_to: AddTo | None = None):
     """x[M, K] . w[N, K]^T (+ bias), accumulated in float. ``out_dtype`` may be
-    float32 for bfloat16 inputs (the logits)."""
+    float32 for bfloat16 inputs (the logits).
+    ``x`` may be a ``Normed``: where the product's kernel can, it scales the rows itself.
+    ``add_to``: the residual stream [M, N] that the caller is about to add the result to, and the norm that follows.
+    Where the product's kernel can, it makes the addition itself (in float; the stream is rewritten) and a ``Summed``
+    is returned, which that norm takes; otherwise the plain result is returned and the stream is left alone."""
+    normed = x if isinstance(x, Normed) else None
+    if normed is not None:
+        x = normed.summed.weighted
+        _dense(w, "linear: w", dtype=x.dtype)
+        if not (_may_fuse(x, w) and _fusion_pays(x, w, False)):
+            x, normed = normed.tensor(), None
     _need(x.dim() == 2 and w.dim() == 2, "linear: x must be [rows, in] and w [out, in]")
     _need(x.shape[1] == w.shape[1], lambda: f"linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
     _dense(x, "linear: x")
@@ -700,14 +881,39 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, o
         _dense(bias, "linear: bias", (w.shape[0],), x.dtype)
     out_dtype = out_dtype or x.dtype
     _need(out_dtype == x.dtype or out_dtype == torch.float32, lambda: f"linear: output of {out_dtype} from {x.dtype}")
-    out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
-    backend().linear(x, w, bias, out)
+    M, N = x.shape[0], w.shape[0]
+    scales = None if normed is None else (normed.summed.squares, float(normed.summed.eps))
+    if add_to is not None and out_dtype == x.dtype and _may_fuse(x, w) and (normed is not None or _addition_pays(x, w, add_to)):
+        residual = add_to.residual
+        _dense(residual, "linear: residual", (M, N))
+        _need(residual.dtype == x.dtype or residual.dtype == torch.float32, lambda: f"linear: residual of {residual.dtype} with rows of {x.dtype}")
+        _dense(add_to.norm_weight, "linear: the next norm's weight", (N,))
+        dtype_code(add_to.norm_weight)
+        weighted = torch.empty((M, N), dtype=x.dtype, device=x.device)
+        squares = torch.empty((M, (N + 15) // 16), dtype=torch.float32, device=x.device)
+        backend().fused_linear(x, w, bias, None, row_scales=scales, residual=residual, sum_out=weighted, ss_out=squares,
+                               next_w=add_to.norm_weight)
+        return Summed(weighted, squares, residual, add_to.norm_weight, add_to.eps)
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if normed is not None:
+        backend().fused_linear(x, w, bias, out, row_scales=scales)
+    else:
+        backend().linear(x, w, bias, out)
     return out
 
 
-def gated_linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+def gated_linear(x, w: torch.Tensor) -> torch.Tensor:
     """silu(x . w[:I]^T) * (x . w[I:]^T) for a packed gate | up matrix w[2 I, K]: fused into one kernel for
-    few rows, else the matrix product followed by ``silu_mul``."""
+    few rows, else the matrix product followed by ``silu_mul``. ``x`` may be a ``Normed`` (see ``linear``)."""
+    if isinstance(x, Normed):
+        normed, x = x, x.summed.weighted
+        _need(w.dim() == 2 and w.shape[0] % 2 == 0 and x.shape[1] == w.shape[1], "gated_linear: w must be [2 * out, in]")
+        _dense(w, "gated_linear: w", dtype=x.dtype)
+        if _may_fuse(x, w) and _fusion_pays(x, w, True):
+            out = torch.empty((x.shape[0], w.shape[0] // 2), dtype=x.dtype, device=x.device)
+            backend().fused_linear(x, w, None, out, gated=True, row_scales=(normed.summed.squares, float(normed.summed.eps)))
+            return out
+        x = normed.tensor()
     _need(x.dim() == 2 and w.dim() == 2 and w.shape[0] % 2 == 0, "gated_linear: x must be [rows, in] and w [2 * out, in]")
     _need(x.shape[1] == w.shape[1], lambda: f"gated_linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
     _dense(x, "gated_linear: x")

@@ -25,5 +25,12 @@ class SwiGLU(Part):
             "down.weight": ParamSpec((self.hidden_size, self.intermediate_size)),
         }
 
-    def forward(self, x: torch.Tensor, step) -> torch.Tensor:
-        return ops.linear(ops.gated_linear(x, self.gate_up_weight), self.down_weight)
+    takes_deferred_norm = True    # x goes straight into a product, which can norm it
+    adds_to_residual = True       # the down projection can make the addition to the residual stream
+
+    def first_product(self):
+        """(weight, gated) of the product that x goes into."""
+        return self.gate_up_weight, True
+
+    def forward(self, x, step, add_to=None):
+        return ops.linear(ops.gated_linear(x, self.gate_up_weight), self.down_weight, add_to=add_to)

@@ -58,7 +58,14 @@ class GQAAttention(Part):
     def cache_need(self):
         return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x: torch.Tensor, step, cache: CacheView) -> torch.Tensor:
+    takes_deferred_norm = True    # x goes straight into a product, which can norm it
+    adds_to_residual = True       # the output projection can make the addition to the residual stream
+
+    def first_product(self):
+        """(weight, gated) of the product that x goes into."""
+        return self.qkv_weight, False
+
+    def forward(self, x, step, cache: CacheView, add_to=None):
         tables = step.groups[cache.group]
         qkv = ops.linear(x, self.qkv_weight)
         # an encoding over several position axes says which axis turns each pair; others turn by the first axis
@@ -70,4 +77,4 @@ class GQAAttention(Part):
             tables.slot_mapping, cache.k, cache.v, self.num_heads, self.num_kv_heads, self.head_dim,
             write_kv=cache.writes, pair_axes=pair_axes)
         o = ops.paged_attention(q, cache.k, cache.v, step.attention, tables.block_tables, self.scale, self.window)
-        return ops.linear(o.view(o.shape[0], self.num_heads * self.head_dim), self.o_weight)
+        return ops.linear(o.view(o.shape[0], self.num_heads * self.head_dim), self.o_weight, add_to=add_to)

@@ -160,11 +160,27 @@ class DecoderModel(Part):
         """Hidden states after the final norm, for the rows whose logits are wanted only: [n, hidden]."""
         hidden = ops.embed(step.input_ids, self.embed_weight, self.spec.embed_scale)
         residual = None
-        for entry, cache in zip(self.run_order, self.cache_views):
-            hidden, residual = self.layers[entry.layer].forward(hidden, residual, step, cache)
+        order = self.run_order
+        for i, (entry, cache) in enumerate(zip(order, self.cache_views)):
+            layer = self.layers[entry.layer]
+            # a block that knows ``ops.Summed`` (a sum that a product has made already, in place of a tensor still to be
+            # added) may hand one on to the norm that comes next, if that knows it too: the next block's first norm, or
+            # this model's last
+            more = {}
+            if getattr(layer, "takes_summed", False):
+                if i + 1 == len(order):
+                    more["next_norm"] = self.final_norm if getattr(self.final_norm, "takes_summed", False) else None
+                else:
+                    nxt = self.layers[order[i + 1].layer]
+                    if getattr(nxt, "takes_summed", False):
+                        more["next_norm"], more["next_reader"] = nxt.mixer_norm, nxt.mixer
+            hidden, residual = layer.forward(hidden, residual, step, cache, **more)
         if step.num_logit_rows == 0:
             return None
         # only the wanted rows go through the last norm and the head (nanovllm/layers/embed_head.py:56-61)
+        if isinstance(hidden, ops.Summed):    # the last product has added itself to the residual stream already
+            hidden, _ = self.final_norm.forward_add(hidden, residual)
+            return ops.gather_rows(hidden, step.logit_rows)
         hidden = ops.gather_rows(hidden, step.logit_rows)
         if residual is None:                  # the last block has made its additions itself
             return self.final_norm.forward(hidden)

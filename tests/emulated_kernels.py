@@ -102,6 +102,35 @@ class EmulatedBackend:
             y = y + bias.float()
         out.copy_(y.to(out.dtype))
 
+    # products of few rows that take over the residual addition after them and the norm before them
+    few_rows = 16
+    fuse_norms = True
+
+    def fused_linear(self, x, w, bias, out, gated=False, row_scales=None, residual=None, sum_out=None, ss_out=None, next_w=None):
+        dt = x.dtype
+        y = x.float() @ w.float().T
+        if row_scales is not None:
+            ss, eps = row_scales
+            y = y * torch.rsqrt(ss.sum(-1, keepdim=True) / x.shape[1] + eps)
+        if gated:
+            half = w.shape[0] // 2
+            g, u = y[:, :half], y[:, half:]
+            y = g * torch.sigmoid(g) * u
+        elif bias is not None:
+            y = y + bias.float()
+        if residual is None:
+            out.copy_(y.to(out.dtype))
+            return
+        s = y + residual.float()
+        residual.copy_(s.to(residual.dtype))
+        sum_out.copy_((s * (next_w.float() if next_w is not None else 1.0)).to(dt))
+        pad = (-s.shape[1]) % 16
+        ss_out.copy_(torch.nn.functional.pad(s * s, (0, pad)).view(s.shape[0], -1, 16).sum(-1))
+
+    def scale_rows(self, x, squares, eps, out):
+        r = torch.rsqrt(squares.sum(-1, keepdim=True) / x.shape[1] + eps)
+        out.copy_((x.float() * r).to(out.dtype))
+
     def sample(self, logits, temperatures, keys, tokens):
         from plain_qwen3 import sample_token
         import math

@@ -382,12 +382,23 @@ def test_pinned_gemm_choices_make_bfloat16_runs_repeat_bit_for_bit(model_folders
     assert json.load(open(path)) == table
     backend.chosen.clear()
     llm = LLM(folder, gemm_choices=path, **options)
-    assert backend.measuring_allowed is False and llm.gemm_choices() == table
+    assert llm.gemm_choices() == table
+    # a second engine of the same process, which measures and keeps the process-wide table, steps in between:
+    # neither changes how the other's products are done
+    other = LLM(folder, **options)
+    assert other.runner.gemm_table is None and other.runner.measure_gemms
+    logits_of(other)
     again = logits_of(llm)
+    assert backend.measuring_allowed is False and backend.chosen is llm.runner.gemm_table
     assert llm.gemm_choices() == table, "nothing was measured in the second run"
     assert torch.equal(again, measured)
-    backend.measuring_allowed = True
-    backend.chosen.clear()
+    logits_of(other)
+    assert backend.measuring_allowed is True and backend.chosen is backend.shared_chosen
+    # a table that names an algorithm the library does not have is refused when the engine starts
+    bad = str(tmp_path / "bad.json")
+    json.dump({"8,512,512,0,0": 100000}, open(bad, "w"))
+    with pytest.raises(Exception, match="algorithms for this shape"):
+        LLM(folder, gemm_choices=bad, **options)
 
 
 @pytest.mark.gpu

@@ -118,6 +118,69 @@ def test_linear(ops, dtype, M, N, K):
         torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32).double(), ref, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("residual_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("norm_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,H,N", [(1, 4096, 6144), (8, 4096, 1536), (16, 1024, 389), (5, 96, 80), (16, 12288, 512), (7, 5120, 4096)])
+def test_products_that_take_over_the_addition_and_the_norm(ops, M, H, N, norm_dtype, residual_dtype):
+    """``linear(x, w, add_to=AddTo(residual, norm weight, eps))`` of few rows adds its result to the residual stream
+    in its own kernel and leaves the sum times the norm's weight, rounded, and the tiles' shares of the rows' sums
+    of squares (``Summed``); what is left of the norm, the scaling of the rows, is done by the product that reads
+    ``Normed(summed)``, on its finished sums. Both against the same steps in float64: residual += x w1^T;
+    y = rmsnorm(residual) w2^T (plain and gated)."""
+    K1 = 256
+    x = rnd(M, K1, dtype=torch.bfloat16, seed=31)
+    w1 = rnd(H, K1, dtype=torch.bfloat16, seed=32, scale=K1 ** -0.5)
+    residual = rnd(M, H, dtype=residual_dtype, seed=33)
+    before = residual.clone()
+    norm_w = (1 + 0.1 * torch.randn(H)).to(norm_dtype).cuda()
+    w2 = rnd(N, H, dtype=torch.bfloat16, seed=34, scale=H ** -0.5)
+    w3 = rnd(2 * (N // 2), H, dtype=torch.bfloat16, seed=35, scale=H ** -0.5)
+    bias = rnd(N, dtype=torch.bfloat16, seed=37)
+    eps = 1e-5
+    summed = ops.linear(x, w1, add_to=ops.AddTo(residual, norm_w, eps))
+    assert isinstance(summed, ops.Summed) and summed.residual is residual and summed.norm_weight is norm_w
+    want_sum = before.double() + x.double() @ w1.double().T
+    torch.testing.assert_close(residual.double(), want_sum, **(dict(rtol=1e-5, atol=1e-5) if residual_dtype == torch.float32 else tol(torch.bfloat16)))
+    torch.testing.assert_close(summed.weighted.double(), want_sum * norm_w.double(), **tol(torch.bfloat16))
+    assert summed.squares.shape == (M, (H + 15) // 16)
+    torch.testing.assert_close(summed.squares.double().sum(-1), want_sum.pow(2).sum(-1), rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(summed.squares[:, 3].double(), want_sum[:, 48:64].pow(2).sum(-1), rtol=1e-4, atol=1e-4)
+    # the scaling left to the products that read it
+    normed = ops.Normed(summed)
+    scale = torch.rsqrt(want_sum.pow(2).mean(-1, keepdim=True) + eps)
+    want_normed = want_sum * scale * norm_w.double()
+    torch.testing.assert_close(normed.tensor().double(), want_normed, **tol(torch.bfloat16))
+    # (the products are compared with products of the weighted sum as it was rounded, scaled afterwards: what is left
+    # is the order of the sums)
+    rows = summed.weighted.double()
+    y = ops.linear(normed, w2, bias)
+    torch.testing.assert_close(y.double(), rows @ w2.double().T * scale + bias.double(), **tol(torch.bfloat16))
+    torch.testing.assert_close(y.double(), want_normed @ w2.double().T + bias.double(), rtol=3e-2, atol=3e-2)
+    g = rows @ w3.double().T * scale
+    half = w3.shape[0] // 2
+    torch.testing.assert_close(ops.gated_linear(normed, w3).double(),
+                               torch.nn.functional.silu(g[:, :half]) * g[:, half:], **tol(torch.bfloat16))
+    # and one product that does both: the scaling of its rows and the addition of its result
+    res2 = rnd(M, N, dtype=residual_dtype, seed=36)
+    before2 = res2.clone()
+    next_w = (1 + 0.1 * torch.randn(N)).to(norm_dtype).cuda()
+    both = ops.linear(normed, w2, add_to=ops.AddTo(res2, next_w, eps))
+    assert isinstance(both, ops.Summed)
+    torch.testing.assert_close(both.weighted.double(), (before2.double() + rows @ w2.double().T * scale) * next_w.double(),
+                               **tol(torch.bfloat16))
+    # switched off, the same calls give tensors and leave the residual alone
+    backend = ops.backend()
+    backend.fuse_norms = False
+    try:
+        res3 = before.clone()
+        plain = ops.linear(x, w1, add_to=ops.AddTo(res3, norm_w, eps))
+        assert isinstance(plain, torch.Tensor) and torch.equal(res3, before)
+        torch.testing.assert_close(plain.double(), x.double() @ w1.double().T, **tol(torch.bfloat16))
+        torch.testing.assert_close(ops.linear(normed, w2).double(), want_normed @ w2.double().T, rtol=3e-2, atol=3e-2)
+    finally:
+        backend.fuse_norms = True
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 1000, 12288), (16, 389, 96), (17, 301, 80), (33, 6144, 1024),
                                    (48, 50, 2048), (64, 151936, 256), (64, 4096, 12288)])
 def test_skinny_linear_bfloat16(ops, M, N, K):
