@@ -582,12 +582,11 @@ class ModelRunner:
 
     def _use_own_choices(self) -> None:
         """This engine's table of matrix-product choices, and its leave to time, are the ones in force from here on."""
-        if self.device.type == "cuda":
-            from ..native import ops
-            backend = ops.backend()
-            if hasattr(backend, "use_choices"):
-                backend.use_choices(self.gemm_table, self.measure_gemms)
-                backend.fuse_norms = self.fuse_norms
+        from ..native import ops
+        backend = ops.backend()
+        backend.fuse_norms = self.fuse_norms
+        if self.device.type == "cuda" and hasattr(backend, "use_choices"):
+            backend.use_choices(self.gemm_table, self.measure_gemms)
 
     def _poison(self, given_back: list[list[int]]) -> None:
         if not self.poison_freed_pages or not any(given_back):

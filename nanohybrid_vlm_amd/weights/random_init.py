@@ -67,10 +67,12 @@ def write_random_model(folder: str, raw_config: dict, seed: int, store_dtype: st
     return folder
 
 
-def fill_random_on_device(model, seed: int, dtype: torch.dtype, device) -> dict[str, torch.Tensor]:
+def fill_from_device_generator(model, seed: int, dtype: torch.dtype, device) -> dict[str, torch.Tensor]:
     """The same distributions drawn straight into the model's parameters on the
-    device, for measurements at sizes whose files would take minutes to write.
-    (The numbers differ from ``write_random_model``'s for the same seed.)"""
+    device by the device's own generator, for measurements at sizes whose files would take
+    minutes to write. These are other numbers than ``write_random_model`` writes for the same
+    seed (another generator, one stream for all tensors): a model made this way is compared with
+    nothing but itself."""
     gen = torch.Generator(device=device)
     gen.manual_seed(int(seed))
     params = {}
@@ -89,7 +91,8 @@ def fill_random_on_device(model, seed: int, dtype: torch.dtype, device) -> dict[
 def build_random_model(raw_config: dict, seed: int, dtype: str | torch.dtype = "bfloat16", device="cuda:0",
                        options: dict | None = None):
     """(architecture, typed configuration, model with random weights bound) from config.json contents: what
-    ``ModelRunner`` and ``LLM`` take in place of a model folder. The weights are drawn on the device.
+    ``ModelRunner`` and ``LLM`` take in place of a model folder. The weights are drawn on the device
+    (``fill_from_device_generator``: not the numbers that a folder of the same seed holds).
     ``options``: engine options offered to the parts' constructors (see ``DecoderModel``)."""
     from ..parts.model import DecoderModel
 
@@ -98,5 +101,5 @@ def build_random_model(raw_config: dict, seed: int, dtype: str | torch.dtype = "
     model = DecoderModel(arch.build_spec(cfg), options=options)
     if isinstance(dtype, str):
         dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}[dtype]
-    fill_random_on_device(model, seed, dtype, device)
+    fill_from_device_generator(model, seed, dtype, device)
     return arch, cfg, model

@@ -582,3 +582,64 @@ def test_short_step_graphs_stay_within_the_models_positions(model_folders):
     got = rc.run_in_process(runner, [{"step": 0, "entries": [{"id": "a", "tokens": tokens, "want": [39]}], "end": ["a"]}])
     assert runner.get_memory_stats()["mixed_graphs_recorded"] == [(48, 1)]
     assert max_abs_diff(got["a"], plain.logits(cfg, w, tokens)[39:]) <= tolerance_for("float32", got)
+
+
+def _decode_logits(folder, device, dtype, fuse, graphs=False):
+    """Six requests decoding side by side after their prompts (steps of up to 16 rows), every logit."""
+    from nanohybrid_vlm_amd.engine.runner import ModelRunner
+    cfg, _ = plain.read_model_folder(folder)
+    requests = {f"r{i}": rc.random_tokens(cfg["vocab_size"], 20 + 3 * i, 700 + i) for i in range(6)}
+    alone = rc.tail_decoded(requests, tail=8)
+    steps = alone + _renamed(rc.mixed(requests, max_live=6, sizes=(3, 2, 5)), "'", len(alone))
+    runner = ModelRunner(folder, dtype=dtype, device=device, page_size=8, num_pages=64, num_state_slots=8, use_graphs=graphs,
+                         max_model_len=128, fuse_norms=fuse)
+    return requests, rc.run_in_process(runner, steps), runner
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_products_take_over_norms_on_emulated_kernels(model_folders, emulated_kernels, name):
+    """In bfloat16 a product of up to 16 rows may make the residual addition after it and leave only the scaling of
+    the rows to the product that reads the norm. With and without, the logits agree within bfloat16's rounding, and
+    with it the work really is taken over (the stand-in's fused product is called, the norm's kernel far less)."""
+    from nanohybrid_vlm_amd.native import ops
+    backend = ops.backend()
+    calls = {"fused": 0, "norm": 0}
+    fused_linear, rmsnorm = backend.fused_linear, backend.rmsnorm
+    backend.fused_linear = lambda *a, **k: (calls.__setitem__("fused", calls["fused"] + 1), fused_linear(*a, **k))[1]
+    backend.rmsnorm = lambda *a, **k: (calls.__setitem__("norm", calls["norm"] + 1), rmsnorm(*a, **k))[1]
+    try:
+        requests, with_fusion, _ = _decode_logits(model_folders[name], "cpu", "bfloat16", True)
+        taken_over = dict(calls)
+        calls.update(fused=0, norm=0)
+        _, without, _ = _decode_logits(model_folders[name], "cpu", "bfloat16", False)
+        plain_way = dict(calls)
+    finally:
+        del backend.fused_linear, backend.rmsnorm
+    assert plain_way["fused"] == 0 and taken_over["fused"] > 0
+    assert taken_over["norm"] < 0.5 * plain_way["norm"], (taken_over, plain_way)
+    want = _plain_logits(model_folders[name], requests)
+    tol = tolerance_for("bfloat16", want)
+    for rid in with_fusion:
+        reference = want[rid.rstrip("'")]
+        assert max_abs_diff(with_fusion[rid], without[rid]) <= tol, rid
+        assert max_abs_diff(with_fusion[rid], reference) <= tol, rid
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_products_take_over_norms_on_gpu(model_folders, name, graphs):
+    """The same on the GPU, for all four small configurations (with and without q/k norms, projection biases, tied
+    heads; head sizes 16 to 128): with the norms taken over and without, against the plain implementation."""
+    folder = model_folders[name]
+    requests, with_fusion, runner = _decode_logits(folder, "cuda:0", "bfloat16", True, graphs)
+    _, without, _ = _decode_logits(folder, "cuda:0", "bfloat16", False, graphs)
+    want = _plain_logits(folder, requests)
+    tol = tolerance_for("bfloat16", want)
+    for rid in with_fusion:
+        reference = want[rid.rstrip("'")]
+        assert max_abs_diff(with_fusion[rid], reference) <= tol, f"taken over, {rid}"
+        assert max_abs_diff(without[rid], reference) <= tol, f"plain, {rid}"
+    if graphs:
+        stats = runner.get_memory_stats()
+        assert stats["graphs_recorded"] and not stats["graphs_refused"] and not stats["mixed_graphs_refused"], stats
