@@ -454,6 +454,62 @@ def test_decode_attention_of_few_tokens_over_many_splits(ops, Hq, Hkv, D, page, 
         torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("D,split_len,n_splits,window", [
+    (128, 64, 5, None),      # one wave, four splits a lane
+    (128, 64, 20, None),     # four waves, four splits a lane; the last waves' splits lie past every position but one
+    (128, 64, 40, 900),      # four waves, eight a lane, a window that leaves the first splits out
+    (128, 64, 100, None),    # four waves, sixteen a lane
+    (128, 64, 140, None),    # past the at-once kernels: the kernel that loops, four waves
+    (64, 128, 9, None), (256, 64, 3, None), (256, 64, 30, 500), (48, 64, 33, None), (16, 64, 70, None),
+])
+def test_merge_of_splits_in_all_its_forms(ops, D, split_len, n_splits, window):
+    """The decode kernel called with the split length and the number of splits named: every form of the merge (one
+    wave or four, 4 to 16 splits a lane, and the looping kernel), with more splits than most positions reach and the
+    buffers of the splits' results full of NaN beforehand, so that a split read without having been written shows."""
+    import ctypes
+    from nanohybrid_vlm_amd.native.ops import _ptr, _stream
+    Hq, Hkv, page = 8, 2, 64
+    longest = n_splits * split_len
+    lens = [longest, 1, split_len, split_len + 1, longest // 2 + 3, longest - 1, 77]
+    lens = [n for n in lens if n <= longest]
+    q_lens = [1] * len(lens)
+    scale = D ** -0.5
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=61, scale=1.5)
+    backend = ops.backend()
+    T = len(lens)
+    out = torch.full((T, Hq, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    part_o = torch.full((T, Hq, n_splits, D), float("nan"), dtype=torch.float32, device="cuda")
+    part_ml = torch.full((T, Hq, n_splits, 2), float("nan"), dtype=torch.float32, device="cuda")
+    backend._call("nhv_decode_attention_bf16", _ptr(q), _ptr(kc), _ptr(vc), _ptr(out), _ptr(part_o), _ptr(part_ml),
+                  _ptr(batch.token_req), _ptr(batch.positions), _ptr(bt), bt.shape[1], T, Hq, Hkv, page,
+                  ctypes.c_float(scale), window or 0, split_len, n_splits, _stream(), lib=backend.attention_lib(D))
+    ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, window)
+    torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
+
+
+def test_merge_of_splits_of_many_tokens(ops):
+    """More than 1,024 (token, head) pairs with more splits than the at-once kernels take: the looping kernel with
+    one wave."""
+    import ctypes
+    from nanohybrid_vlm_amd.native.ops import _ptr, _stream
+    Hq, Hkv, D, page, split_len, n_splits = 16, 2, 128, 64, 64, 140
+    lens = [8960] + [40 + 3 * i for i in range(69)]
+    q_lens = [1] * len(lens)
+    scale = D ** -0.5
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=62, scale=1.5)
+    backend = ops.backend()
+    T = len(lens)
+    assert T * Hq > 1024
+    out = torch.full((T, Hq, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    part_o = torch.full((T, Hq, n_splits, D), float("nan"), dtype=torch.float32, device="cuda")
+    part_ml = torch.full((T, Hq, n_splits, 2), float("nan"), dtype=torch.float32, device="cuda")
+    backend._call("nhv_decode_attention_bf16", _ptr(q), _ptr(kc), _ptr(vc), _ptr(out), _ptr(part_o), _ptr(part_ml),
+                  _ptr(batch.token_req), _ptr(batch.positions), _ptr(bt), bt.shape[1], T, Hq, Hkv, page,
+                  ctypes.c_float(scale), 0, split_len, n_splits, _stream(), lib=backend.attention_lib(D))
+    ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, None)
+    torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("Hq,Hkv,D,page,window", [
     (4, 1, 128, 256, None), (8, 2, 64, 16, None), (6, 1, 32, 8, 100), (3, 3, 48, 5, None), (16, 1, 16, 64, None),
     (5, 1, 256, 32, None), (32, 8, 128, 64, 700),
