@@ -17,6 +17,34 @@ import os
 import torch
 
 
+# Where an engine that computes in bfloat16 stores a result in bfloat16, ``stored`` rounds it to that type and back;
+# by default it does nothing and everything is float32. The reference runs its model in bfloat16 throughout
+# (nanovllm/engine/model_runner.py sets the default dtype from the configuration's torch_dtype), so every
+# layer's output is rounded there: projections, norms, rotated queries and keys, the attention's output
+# (flash-attention also rounds the softmax's weights before the second product), the gated product.
+# The residual sum is kept in float32 here, as the rules of this build ask.
+_STORED_DTYPE = None
+
+
+class stored_as:
+    """``with stored_as(torch.bfloat16): logits(...)``: the same formulas with stored results rounded."""
+
+    def __init__(self, dtype):
+        self.dtype = dtype
+
+    def __enter__(self):
+        global _STORED_DTYPE
+        self.old, _STORED_DTYPE = _STORED_DTYPE, self.dtype
+
+    def __exit__(self, *exc):
+        global _STORED_DTYPE
+        _STORED_DTYPE = self.old
+
+
+def stored(x: torch.Tensor) -> torch.Tensor:
+    return x if _STORED_DTYPE is None else x.to(_STORED_DTYPE).to(torch.float32)
+
+
 def read_model_folder(folder: str):
     """config.json as a dict and every tensor of model.safetensors as float32."""
     from safetensors import safe_open
@@ -35,7 +63,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     dimension, eps inside the square root, weight multiplied last."""
     x = x.to(torch.float32)
     var = x.pow(2).mean(dim=-1, keepdim=True)
-    return x * torch.rsqrt(var + eps) * weight
+    # (layernorm.py:25: the scaled row goes back to the model's type before the weight is multiplied in)
+    return stored(stored(x * torch.rsqrt(var + eps)) * weight)
 
 
 def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float):
@@ -65,7 +94,7 @@ def apply_rope(x: torch.Tensor, positions: torch.Tensor, base: float, rotary_dim
     x1, x2 = xr[..., : d // 2], xr[..., d // 2:]
     y1 = x1 * cos - x2 * sin
     y2 = x2 * cos + x1 * sin
-    return torch.cat((y1, y2, x[..., d:].to(torch.float32)), dim=-1)
+    return stored(torch.cat((y1, y2, x[..., d:].to(torch.float32)), dim=-1))
 
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
@@ -87,16 +116,21 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
         vh = v[:, h // group, :].to(torch.float32)
         scores = (q[:, h, :].to(torch.float32) @ kh.T) * scale
         scores = scores.masked_fill(~allowed, float("-inf"))
-        out[:, h, :] = torch.softmax(scores, dim=-1) @ vh
-    return out
+        if _STORED_DTYPE is None:
+            out[:, h, :] = torch.softmax(scores, dim=-1) @ vh
+        else:
+            # the weights are rounded for the second product; their sum is taken before the rounding
+            e = torch.exp(scores - scores.max(dim=-1, keepdim=True).values)
+            out[:, h, :] = (stored(e) @ vh) / e.sum(dim=-1, keepdim=True)
+    return stored(out)
 
 
 def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
     """nanovllm/models/qwen3.py:113-117 and nanovllm/layers/activation.py:10-11:
     silu(x Wg^T) * (x Wu^T), then the down projection."""
-    g = x @ w_gate.T
-    u = x @ w_up.T
-    return (g * torch.sigmoid(g) * u) @ w_down.T
+    g = stored(x @ w_gate.T)
+    u = stored(x @ w_up.T)
+    return stored(stored(g * torch.sigmoid(g) * u) @ w_down.T)
 
 
 def attention_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: str, cfg: dict) -> torch.Tensor:
@@ -119,6 +153,7 @@ def attention_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: s
         q = q + w[prefix + "q_proj.bias"]
         k = k + w[prefix + "k_proj.bias"]
         v = v + w[prefix + "v_proj.bias"]
+    q, k, v = stored(q), stored(k), stored(v)
     q = q.view(T, Hq, D)
     k = k.view(T, Hkv, D)
     v = v.view(T, Hkv, D)
@@ -128,7 +163,7 @@ def attention_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: s
     q = apply_rope(q, positions, theta)
     k = apply_rope(k, positions, theta)
     o = causal_attention(q, k, v, D ** -0.5)
-    return o.reshape(T, Hq * D) @ w[prefix + "o_proj.weight"].T
+    return stored(o.reshape(T, Hq * D) @ w[prefix + "o_proj.weight"].T)
 
 
 def hidden_states(cfg: dict, w: dict, token_ids, first_position: int = 0) -> torch.Tensor:

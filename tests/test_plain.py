@@ -119,6 +119,29 @@ def test_only_distances_between_positions_count(cfg, seed):
     torch.testing.assert_close(a, b, rtol=1e-4, atol=2e-5)
 
 
+@pytest.mark.parametrize("cfg,seed", [(TINY_A, 0), (TINY_B, 1)])
+def test_stored_results_rounded_to_bfloat16(cfg, seed):
+    """``stored_as(bfloat16)`` rounds where the reference's bfloat16 model stores (nanovllm/layers/layernorm.py:25,
+    rotary_embedding.py:13): the parts' results are then bfloat16 numbers, a norm rounds the scaled row before the
+    weight, the logits move by some bfloat16 roundings and no more, and leaving the block restores float32."""
+    w = _random_weights(cfg, seed)
+    toks = torch.randint(0, cfg["vocab_size"], (23,)).tolist()
+    exact = plain.logits(cfg, w, toks)
+    x = torch.randn(7, 24)
+    weight = 1 + 0.1 * torch.randn(24)
+    with plain.stored_as(torch.bfloat16):
+        rounded = plain.logits(cfg, w, toks)
+        y = plain.rms_norm(x, weight, 1e-6)
+        r = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)
+        assert torch.equal(y, (r.bfloat16().float() * weight).bfloat16().float())
+        assert not torch.equal(y, (r * weight).bfloat16().float())          # (rounding once would differ somewhere)
+        h = plain.hidden_states(cfg, w, toks)
+        assert torch.equal(h, h.bfloat16().float())
+    assert torch.equal(plain.logits(cfg, w, toks), exact)
+    diff = (rounded - exact).abs().max().item()
+    assert 1e-4 < diff < 0.05 * exact.abs().max().item(), diff
+
+
 def test_causality_and_dead_layers():
     cfg = TINY_A
     w = _random_weights(cfg, 0)

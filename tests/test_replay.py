@@ -39,19 +39,12 @@ def _check(got, want, tol, what):
 
 def _rounding_reference(folder, requests):
     """bfloat16 with sharpened attention: rounding q and k to 8 bits moves scores of size 16 by up to 0.06
-    and the logits by several 1e-2, which would hide a lost key. There the reference is the CPU stand-in for
-    the kernels run in bfloat16 (same places of rounding, whole requests, its float32 run is itself checked
-    against the plain implementation), and the tolerance stays that of bfloat16."""
-    from emulated_kernels import EmulatedBackend
-    from nanohybrid_vlm_amd.engine.runner import ModelRunner
-    from nanohybrid_vlm_amd.native import ops
-    old = ops._backend
-    ops.set_backend(EmulatedBackend())
-    try:
-        runner = ModelRunner(folder, dtype="bfloat16", device="cpu", page_size=16, num_pages=16, num_state_slots=2)
-        return rc.run_in_process(runner, rc.whole(requests))
-    finally:
-        ops.set_backend(old)
+    and the logits by several 1e-2, which would hide a lost key. There the reference is the plain implementation
+    with every stored result rounded to bfloat16 (``plain.stored_as``: the same formulas, whole requests, no cache),
+    and the tolerance stays that of bfloat16."""
+    cfg, w = plain.read_model_folder(folder)
+    with plain.stored_as(torch.bfloat16):
+        return {rid: plain.logits(cfg, w, toks) for rid, toks in requests.items()}
 
 
 def _poisoned(runner):
