@@ -371,13 +371,24 @@ __global__ __launch_bounds__(256) void qk_rope_write_vec_kernel(
   const int width = (Hq + 2 * Hkv) * D;
   const bool is_q = h < Hq;
   const bool is_k = !is_q && h < Hq + Hkv;
+  // everything that does not hang on another load is asked for before anything is looked at (a key's or value's
+  // slot used to be waited for before its entries were asked for, one trip to memory after the other)
+  float v[8];
+  load8f<T>(qkv + (size_t)t * width + (size_t)h * D + c * 8, v);
+  const int pos = rot > 0 ? positions[t] : 0;
   int slot = -1;
   if (!is_q) {
     slot = slot_mapping[t];
     if (slot < 0) return;
   }
-  float v[8];
-  load8f<T>(qkv + (size_t)t * width + (size_t)h * D + c * 8, v);
+  constexpr int HALF_LANES = CH / 2 > 0 ? CH / 2 : 1;
+  float cs[8], sn[8];
+  if (rot > 0 && (is_q || is_k)) {
+    const float* row = cos_sin + (size_t)pos * rot;
+    const int j = (c % HALF_LANES) * 8;              // index into the table's cosines; sines lie rot / 2 further
+    load8f<float>(row + j, cs);
+    load8f<float>(row + rot / 2 + j, sn);
+  }
   if (bias) {
     float b[8];
     load8f<T>(bias + (size_t)h * D + c * 8, b);
@@ -403,12 +414,6 @@ __global__ __launch_bounds__(256) void qk_rope_write_vec_kernel(
   }
   float o[8];
   if (rot > 0) {
-    constexpr int HALF_LANES = CH / 2 > 0 ? CH / 2 : 1;
-    float cs[8], sn[8];
-    const float* row = cos_sin + (size_t)positions[t] * rot;
-    const int j = (c % HALF_LANES) * 8;              // index into the table's cosines; sines lie rot / 2 further
-    load8f<float>(row + j, cs);
-    load8f<float>(row + rot / 2 + j, sn);
     const bool first_half = c < HALF_LANES;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
