@@ -120,7 +120,8 @@ def test_linear(ops, dtype, M, N, K):
 
 @pytest.mark.parametrize("residual_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("norm_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("M,H,N", [(1, 4096, 6144), (8, 4096, 1536), (16, 1024, 389), (5, 96, 80), (16, 12288, 512), (7, 5120, 4096)])
+@pytest.mark.parametrize("M,H,N", [(1, 4096, 6144), (8, 4096, 1536), (16, 1024, 389), (5, 96, 80), (16, 12288, 512), (7, 5120, 4096),
+                                   (3, 72, 40), (16, 1000, 24), (12, 2056, 130)])      # widths that end inside a tile of 16
 def test_products_that_take_over_the_addition_and_the_norm(ops, M, H, N, norm_dtype, residual_dtype):
     """``linear(x, w, add_to=AddTo(residual, norm weight, eps))`` of few rows adds its result to the residual stream
     in its own kernel and leaves the sum times the norm's weight, rounded, and the tiles' shares of the rows' sums
