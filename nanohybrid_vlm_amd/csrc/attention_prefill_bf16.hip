@@ -11,7 +11,8 @@
 // what the kernel waits for most); that is taken where the batch still gives every
 // compute unit two blocks of that size. Keys are taken in tiles of 64, in rising order:
 //   S^T[key, row] = K[key, :] . Q[row, :]      K tile from LDS, Q in registers (v_mfma_f32_16x16x32_bf16)
-//   running maximum per row in float (two shuffles over the lane groups), sums kept per lane
+//   exponentials against a reference point per row that moves only when they have outgrown it (then the row's
+//   maximum, two shuffles over the lane groups), sums kept per lane
 //   O^T[d, row]  += V^T[d, key] . P^T[key, row]  V^T from LDS, P in registers (v_mfma_f32_16x16x32_bf16)
 // An S^T tile leaves every lane with four consecutive keys of one row; two such tiles
 // side by side are the eight summation slots of a lane in the second product (the
@@ -253,42 +254,56 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     bool grow[RT];
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
-      // the scale (times log2 e) is positive: the maximum is taken of the raw scores, and the scaling rides in the
-      // multiply-add that also subtracts the reference
-      float m_tile = -INFINITY;
+      // The reference point of a row's exponentials stays where it is as long as they stay far below float's range:
+      // they are taken against it at once, without the tile's maximum, and only a sum that has grown past 2^40 (or is
+      // no number: a row that has seen no key yet has no reference) sends the wave to the maximum and a new reference.
+      if (MASKED) {
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt)
+        for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (MASKED) {
+          for (int j = 0; j < 4; ++j) {
             const int key = kb + kt * 16 + grp * 4 + j;
             if (key > row_pos[r] || key < row_lo[r]) s4[r][kt][j] = -INFINITY;
           }
-          m_tile = fmaxf(m_tile, s4[r][kt][j]);
-        }
-      m_tile *= scale_log2e;
-      // The running maximum is only a reference point: as long as no row of the wave has grown by more than 2^6
-      // over its reference, the reference stays and the output needs no rescaling (P stays below 64). Whether
-      // any row has grown shows in the lanes' own maxima; the row's maximum over its four lanes is only needed then.
-      grow[r] = __any(m_tile > m_run[r] + 6.0f);
-      if (grow[r]) {
-        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
-        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
       }
-      const float m_new = grow[r] ? fmaxf(m_run[r], m_tile) : m_run[r];
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
-      alpha[r] = __builtin_amdgcn_exp2f(m_run[r] - m_safe);
       float psum = 0.f;
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s4[r][kt][j], scale_log2e, -m_safe));
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s4[r][kt][j], scale_log2e, -m_run[r]));
           psum += p;
           pa[r][kt / 2][(kt % 2) * 4 + j] = (__bf16)p;
         }
-      l_part[r] = l_part[r] * alpha[r] + psum;
-      m_run[r] = m_new;
+      grow[r] = __any(!(psum < 1.0995116e12f));
+      alpha[r] = 1.0f;
+      if (grow[r]) {
+        asm volatile("" ::: "memory");
+        float m_tile = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) m_tile = fmaxf(m_tile, s4[r][kt][j]);
+        m_tile *= scale_log2e;
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+        const float m_new = fmaxf(m_run[r], m_tile);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a row that has still seen no key
+        alpha[r] = m_run[r] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[r] - m_safe);
+        psum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s4[r][kt][j], scale_log2e, -m_safe));
+            psum += p;
+            pa[r][kt / 2][(kt % 2) * 4 + j] = (__bf16)p;
+          }
+        l_part[r] = l_part[r] * alpha[r] + psum;
+        m_run[r] = m_new;
+      } else {
+        l_part[r] += psum;
+      }
     }
     // The outputs are rescaled only when a reference has moved: a branch of the whole wave, taken rarely. (Written
     // as a condition inside the loop over the output tiles, the compiler made a multiply and a select of it for

@@ -527,6 +527,32 @@ def test_prefill_attention_bfloat16(ops, Hq, Hkv, D, page, window):
     torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("far", [3, 650, 1290])
+def test_prefill_attention_scores_that_outgrow_their_reference(ops, far):
+    """The prompt kernel takes a row's exponentials against a reference point that stays while they stay far below
+    float's range. Here one key's scores stand 110 powers of two above all others, for every query of one head: an
+    early key (everything after it is tiny against the reference), a key in the middle of the portion and one near
+    its end (the sums so far have to be scaled down by 2^-110 when it comes). Against the float64 computation."""
+    Hq, Hkv, D, page = 4, 2, 128, 64
+    scale = D ** -0.5
+    lens, q_lens = [1300, 200], [700, 200]
+    q, kc, vc, batch, bt, ks, vs, qs = _paged_setup(torch.bfloat16, lens, q_lens, Hq, Hkv, D, page, seed=71, scale=1.0)
+    g = torch.Generator().manual_seed(6)
+    direction = torch.randn(D, generator=g)
+    direction = (direction / direction.norm()).to(torch.bfloat16)
+    ks[0][far, 0] = 30.0 * direction                              # heads 0 and 1 read key/value head 0
+    kc[int(bt[0, far // page]), far % page, 0] = ks[0][far, 0].cuda()
+    qs[0][:, 1] = qs[0][:, 1] + 29.0 * direction                  # 30 x 29 / sqrt(128) = 77 = 111 powers of two
+    q[:q_lens[0], 1] = qs[0][:, 1].cuda()
+    out = ops.paged_attention(q, kc, vc, batch, bt, scale, None)
+    ref = _attention_reference(qs, ks, vs, lens, q_lens, scale, None)
+    torch.testing.assert_close(out.double().cpu(), ref, **tol(torch.bfloat16))
+    # (the input does what it is meant to: a query of head 1 that sees the key puts all of its weight on it)
+    first_q = lens[0] - q_lens[0]
+    row = max(far - first_q, 0) + 5
+    torch.testing.assert_close(ref[row, 1], vs[0][far, 0].double(), rtol=1e-6, atol=1e-6)
+
+
 @pytest.mark.parametrize("window", [None, 5000])
 def test_attention_over_32768_keys(ops, window):
     """Both bfloat16 attention kernels at 32,768 keys on pages of 256 (128 pages a request, hundreds of splits to
