@@ -206,6 +206,8 @@ class NativeBackend:
         # 512), 512 for 48 and 64 x 2,176 (110 against 118 us with 1,024) and for 16 x 8,192, 1,024 for 32 x 8,192.
         want = max(1, T * Hkv * span // 1024)
         want = min(want, max(256, want * 2 // 3))
+        # (splits of one round of 32 keys for one request of 2,100 keys, 525 waves: 3.64 against 3.66 ms a step; for two
+        # requests 3.77 against 3.75: not taken)
         split_len = 64
         while split_len * 2 <= want and split_len < 1024:
             split_len *= 2
