@@ -15,6 +15,7 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -120,8 +121,9 @@ def build_library(stem: str, source_names: list[str], defines: list[str] | None 
             raise NativeBuildError(f"linking {file_name} failed:\n{proc.stderr[-4000:]}")
         os.replace(tmp_target, target)        # atomic: another process never sees half a file
         # libraries of older sources are of no use any more
+        older = re.compile(re.escape(f"lib{stem}_") + r"[0-9a-f]{16}\.so")     # (not a library whose name begins with this one's)
         for f in os.listdir(out_dir):
-            if f.startswith(f"lib{stem}_") and f.endswith(".so") and f != file_name:
+            if older.fullmatch(f) and f != file_name:
                 try:
                     os.remove(os.path.join(out_dir, f))
                 except OSError:
